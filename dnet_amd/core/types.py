@@ -80,4 +80,5 @@ class ShardLoadModelRequest(BaseModel):
     max_batch: int = 8
     max_seq: int = 4096
     quant: str = ""                   # "" | "int8-g128" | ...
+    dtype: str = "bfloat16"           # "float32": true-fp32 compute path
     warmup: bool = False

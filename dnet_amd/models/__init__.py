@@ -39,5 +39,9 @@ from .deepseek_v2 import DeepseekV2RingModel  # noqa: E402
 
 register(DeepseekV2RingModel)
 
-__all__ = ["ModelConfig", "QuantConfig", "RingModel", "MoERingModel", "KVCache",
+from .posudra import PosudraRingModel  # noqa: E402
+
+register(PosudraRingModel)
+
+__all__ = ["ModelConfig", "QuantConfig", "RingModel", "MoERingModel", "KVCache", "PosudraRingModel",
            "Linear", "PRESETS", "get_ring_model", "register"]

@@ -124,6 +124,13 @@ class Linear:
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
         m = x.shape[0]
+        if self.w.dtype == torch.float32:
+            # true-fp32 models: the vendor fp32 GEMM at every M (no
+            # reduced-precision matrix mode is enabled anywhere)
+            y = x @ self.w.t()
+            if self.bias is not None:
+                y = y + self.bias
+            return y
         if self.mxfp4:
             wd, self._wd = (self._wd, None) if self._wd is not None \
                 else (self.dequant(), None)
@@ -131,7 +138,7 @@ class Linear:
             if self.bias is not None:
                 y = y + self.bias
             return y
-        if m <= GEMV_MAX_M:
+        if m <= GEMV_MAX_M and (self.is_quant or self.in_features % 8 == 0):
             self._wd = None
             if self.bits == 4:
                 return ops.gemv_int4(x, self.w, self.scales, self.group,
@@ -173,8 +180,11 @@ class LayerWeights:
     sinks: Optional[torch.Tensor] = None    # gpt-oss attention sinks [Hq]
 
     _TENSOR_FIELDS = ("attn_norm", "mlp_norm", "q_norm", "k_norm", "sinks",
-                      "q_a_norm", "kv_a_norm", "router_bias")
-    _LINEAR_FIELDS = ("qkv", "o", "gateup", "down", "router",
+                      "q_a_norm", "kv_a_norm", "router_bias",
+                      # posudra: per-head score modifiers, activation
+                      # parameters, layer scales
+                      "temp", "dist_r1", "dist_r2", "act_pq", "ls1", "ls2")
+    _LINEAR_FIELDS = ("qkv", "o", "gateup", "down", "router", "up",
                       "shared_gateup", "shared_down", "shared_gate",
                       "q", "q_a", "q_b", "kv_a", "kv_b")
 
@@ -271,11 +281,27 @@ class KVCache:
     """
 
     def __init__(self, cfg: ModelConfig, layer_ids: Sequence[int], batch: int,
-                 smax: int, device, kv_bits: int = 16):
+                 smax: int, device, kv_bits: int = 16,
+                 layer_dims: Optional[Sequence[tuple]] = None,
+                 dtype: torch.dtype = torch.bfloat16):
         self.layer_ids = list(layer_ids)
         self.local = {g: i for i, g in enumerate(self.layer_ids)}
         self.kv_bits = kv_bits
         L = len(self.layer_ids)
+        self.pos = torch.zeros(batch, dtype=torch.int32, device=device)
+        self.smax = smax
+        self.batch = batch
+        self.kscale = self.vscale = None
+        if layer_dims is not None:
+            # heterogeneous stacks: one (kv_heads, k_dim, v_dim) per local
+            # layer -> per-layer tensors [B, Hkv_l, Smax, D_l] (self.k[li]
+            # indexes a list instead of a stacked tensor's first axis)
+            assert kv_bits == 16 and len(layer_dims) == L
+            self.k = [torch.zeros(batch, hk, smax, dk, dtype=dtype,
+                                  device=device) for hk, dk, _ in layer_dims]
+            self.v = [torch.zeros(batch, hk, smax, dv, dtype=dtype,
+                                  device=device) for hk, _, dv in layer_dims]
+            return
         shape = (L, batch, cfg.num_kv_heads, smax, cfg.head_dim)
         if kv_bits == 8:
             ng = cfg.head_dim // 64
@@ -288,9 +314,6 @@ class KVCache:
             self.k = torch.zeros(shape, dtype=torch.bfloat16, device=device)
             self.v = torch.zeros_like(self.k)
             self.kscale = self.vscale = None
-        self.pos = torch.zeros(batch, dtype=torch.int32, device=device)
-        self.smax = smax
-        self.batch = batch
 
     def slot(self, s: int) -> "KVCache":
         """A batch-1 VIEW of slot ``s`` (shared storage): the serving slot
@@ -298,6 +321,12 @@ class KVCache:
         their state (continuous batching)."""
         import copy
         c = copy.copy(self)
+        if isinstance(self.k, list):
+            c.k = [t[s:s + 1] for t in self.k]
+            c.v = [t[s:s + 1] for t in self.v]
+            c.pos = self.pos[s:s + 1]
+            c.batch = 1
+            return c
         c.k = self.k[:, s:s + 1]
         c.v = self.v[:, s:s + 1]
         if getattr(self, "kscale", None) is not None:
@@ -307,9 +336,32 @@ class KVCache:
         c.batch = 1
         return c
 
+    def grow(self, batch: int) -> None:
+        """Add empty slots (rows) up to ``batch``; live rows keep their
+        contents and positions."""
+        extra = batch - self.batch
+        if extra <= 0:
+            return
+
+        def pad(t, axis):
+            shape = list(t.shape)
+            shape[axis] = extra
+            return torch.cat([t, torch.zeros(shape, dtype=t.dtype,
+                                             device=t.device)], dim=axis)
+        if isinstance(self.k, list):
+            self.k = [pad(t, 0) for t in self.k]
+            self.v = [pad(t, 0) for t in self.v]
+        else:
+            self.k, self.v = pad(self.k, 1), pad(self.v, 1)
+            if self.kscale is not None:
+                self.kscale = pad(self.kscale, 1)
+                self.vscale = pad(self.vscale, 1)
+        self.pos = pad(self.pos, 0)
+        self.batch = batch
+
     @property
     def quantized(self) -> bool:
-        return self.k.dtype == torch.int8
+        return (not isinstance(self.k, list)) and self.k.dtype == torch.int8
 
     def k_deq(self, li: int) -> torch.Tensor:
         if not self.quantized:
@@ -327,6 +379,8 @@ class KVCache:
         self.pos.zero_()
 
     def nbytes(self) -> int:
+        if isinstance(self.k, list):
+            return sum(t.numel() * t.element_size() for t in self.k + self.v)
         n = 2 * self.k.numel() * self.k.element_size()
         if self.kscale is not None:
             n += 2 * self.kscale.numel() * self.kscale.element_size()
@@ -427,10 +481,7 @@ class RingModel:
         self.embed: Optional[torch.Tensor] = None
         self.final_norm: Optional[torch.Tensor] = None
         self.lm_head: Optional[Linear] = None
-        cos, sin = ops.rope_tables(smax, cfg.head_dim, cfg.rope_theta,
-                                   scaling=cfg.rope_scaling)
-        self.cos = cos.to(self.device)
-        self.sin = sin.to(self.device)
+        self._init_positional()
         # offload policy hook: when set, layer weights come from the
         # windowed weight cache instead of self.layers
         self.weight_provider = None  # Callable[[int], LayerWeights] | None
@@ -445,6 +496,22 @@ class RingModel:
         # config-only dead weight)
         self._obs_every = obs.sync_every_n if obs.enabled else 0
         self._obs_count = 0
+
+    # dtype of the residual stream this model's windows take and return
+    # (executor buffers and ring hops follow it) and of its logits
+    act_dtype = torch.bfloat16
+    logits_dtype = torch.bfloat16
+    supports_float32 = False      # cfg.compute_dtype == "float32" honoured
+    # prefill_window accepts per-row start positions / lengths (ragged
+    # batches of unequal prompts in one call)
+    ragged_prefill = False
+
+    def _init_positional(self):
+        c = self.cfg
+        cos, sin = ops.rope_tables(self.smax, c.head_dim, c.rope_theta,
+                                   scaling=c.rope_scaling)
+        self.cos = cos.to(self.device)
+        self.sin = sin.to(self.device)
 
     def _layer(self, lid: int) -> "LayerWeights":
         # resident layers win (partial offload keeps non-uniform layers —

@@ -64,13 +64,60 @@ class ModelConfig:
     routed_scaling_factor: float = 1.0
     norm_topk_prob: bool = False
     quant: Optional[QuantConfig] = None
+    # heterogeneous layer stacks (posudra): one dict per layer with its
+    # mixer type + sizes and its feed-forward (None = no feed-forward);
+    # num_q_heads / head_dim / ... above then hold layer 0's sizes
+    layer_specs: Optional[list] = None
+    embedding_scale: float = 1.0
+    # "bfloat16": bf16 weights/activations with 32-bit accumulation;
+    # "float32": weights, activations and matrix products in true fp32
+    # (honoured by the model families that implement it)
+    compute_dtype: str = "bfloat16"
 
     @property
     def qkv_out(self) -> int:
         return (self.num_q_heads + 2 * self.num_kv_heads) * self.head_dim
 
     @classmethod
+    def from_posudra(cls, cfg: dict,
+                     quant: Optional[QuantConfig] = None) -> "ModelConfig":
+        """Posudra checkpoints describe themselves layer by layer:
+        {"architecture": "Posudra", "vocab", "width", "norm": {"eps"},
+        "embedding": {"scale"}, "layers": [{"type", "mixer": {...},
+        "mlp": {...} | null}, ...]}. Every size is per layer."""
+        specs = [dict(s) for s in cfg["layers"]]
+        for i, s in enumerate(specs):
+            if s.get("type") != "attention":
+                raise ValueError(f"posudra layer {i}: unknown mixer type "
+                                 f"{s.get('type')!r}")
+            ff = s.get("mlp")
+            if ff is not None and ff.get("kind", "dense") != "dense":
+                raise ValueError(f"posudra layer {i}: unknown feed-forward "
+                                 f"kind {ff.get('kind')!r}")
+        m0 = specs[0]["mixer"]
+        ffs = [s["mlp"]["ff"] for s in specs if s.get("mlp") is not None]
+        return cls(
+            model_type="posudra",
+            hidden_size=cfg["width"],
+            num_layers=len(specs),
+            num_q_heads=m0["heads"],
+            num_kv_heads=m0["kv_heads"],
+            head_dim=m0["dim"],
+            v_head_dim=m0["vdim"],
+            intermediate_size=max(ffs) if ffs else 0,
+            vocab_size=cfg["vocab"],
+            rms_eps=cfg["norm"]["eps"],
+            embedding_scale=float((cfg.get("embedding") or {}).get("scale",
+                                                                   1.0)),
+            layer_specs=specs,
+            quant=quant,
+        )
+
+    @classmethod
     def from_hf(cls, cfg: dict, quant: Optional[QuantConfig] = None) -> "ModelConfig":
+        if str(cfg.get("architecture", "")).lower() == "posudra" \
+                or cfg.get("model_type") == "posudra":
+            return cls.from_posudra(cfg, quant)
         mt = cfg.get("model_type", "llama")
         hidden = cfg["hidden_size"]
         nq = cfg.get("num_attention_heads", 32)

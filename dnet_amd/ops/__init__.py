@@ -431,3 +431,77 @@ def attn_combine(partials: torch.Tensor,
         _native().attn_combine(partials.contiguous().view(-1), sinks, out, S)
         return out
     return ref.attn_combine(partials, sinks)
+
+
+# ---- fp32-residual / score-modified attention family (posudra) ----
+# Residual stream and every statistic in fp32; activations in the model's
+# compute dtype (bf16 or fp32). Kernels: csrc/resid_f32.hip.cpp,
+# csrc/attn_mod.hip.cpp.
+
+def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    if x.is_cuda:
+        y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _native().rmsnorm_rows(x.contiguous(), w, y, eps)
+        return y
+    return ref.rmsnorm_rows(x, w, eps, out_dtype)
+
+
+def ls_resid_rmsnorm(h: torch.Tensor, a: torch.Tensor, s1: torch.Tensor,
+                     b: torch.Tensor | None, s2: torch.Tensor | None,
+                     wn: torch.Tensor | None, eps: float,
+                     out_dtype: torch.dtype) -> torch.Tensor | None:
+    """h (fp32, in place) += s1*a (+ s2*b); returns rms(h)*wn (or None
+    when wn is None) — one kernel per layer boundary."""
+    if h.is_cuda:
+        assert h.dtype == torch.float32 and h.is_contiguous()
+        y = (torch.empty(h.shape, dtype=out_dtype, device=h.device)
+             if wn is not None else None)
+        _native().ls_resid_rmsnorm(h, a, s1, b, s2, wn, y, eps)
+        return y
+    return ref.ls_resid_rmsnorm(h, a, s1, b, s2, wn, eps, out_dtype)
+
+
+def xielu(z: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
+    if z.is_cuda:
+        y = torch.empty_like(z)
+        _native().xielu(z, pq, y)
+        return y
+    return ref.xielu(z, pq)
+
+
+def qknorm_append(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor,
+                  eps: float, nq: int, nkv: int, d: int, dv: int,
+                  kcache: torch.Tensor, vcache: torch.Tensor,
+                  pos: torch.Tensor, T: int, lens=None, slots=None,
+                  per_head: bool = False) -> torch.Tensor:
+    if qkv.is_cuda:
+        q = torch.empty(qkv.shape[0], nq * d, dtype=qkv.dtype,
+                        device=qkv.device)
+        _native().qknorm_append(qkv, qw, kw, q, kcache, vcache, pos, lens,
+                                slots, eps, nq, nkv, d, dv, T, per_head)
+        return q
+    return ref.qknorm_append(qkv, qw, kw, eps, nq, nkv, d, dv, kcache,
+                             vcache, pos, T, lens, slots, per_head)
+
+
+def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+             pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
+             temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
+             sinks=None, window: int = 0) -> torch.Tensor:
+    """Causal attention against the cache with per-head temperature, tanh
+    soft cap, logarithmic distance penalty and a sink in the softmax
+    denominator (each optional). One entry point for decode (T=1) and
+    ragged batched prefill (T = padded length, lens = real lengths)."""
+    if q.is_cuda:
+        Hkv, D = kcache.shape[1], kcache.shape[3]
+        Dv = vcache.shape[3]
+        Hq = q.shape[1] // D
+        out = torch.empty(q.shape[0], Hq * Dv, dtype=q.dtype,
+                          device=q.device)
+        _native().attn_mod(q, kcache, vcache, pos, lens, slots, out, T,
+                           scale, temp, softcap or 0.0, dist_r1, dist_r2,
+                           sinks, window or 0)
+        return out
+    return ref.attn_mod(q, kcache, vcache, pos, T, scale, lens, slots, temp,
+                        softcap, dist_r1, dist_r2, sinks, window)

@@ -471,3 +471,134 @@ def attn_combine(partials: torch.Tensor,
     num = (acc * w.unsqueeze(-1)).sum(2)
     denom = denom.clamp_min(1e-30)
     return (num / denom.unsqueeze(-1)).to(torch.bfloat16)
+
+
+# ---- fp32-residual / score-modified attention family (posudra) ----
+
+def rmsnorm_rows(x: torch.Tensor, w: torch.Tensor, eps: float,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    """y = x / sqrt(mean(x^2) + eps) * w, statistics in fp32, any in/out
+    dtype (fp32 residual in, bf16 or fp32 activations out)."""
+    xf = x.float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (xf * r * w.float()).to(out_dtype)
+
+
+def ls_resid_rmsnorm(h: torch.Tensor, a: torch.Tensor, s1: torch.Tensor,
+                     b: torch.Tensor | None, s2: torch.Tensor | None,
+                     wn: torch.Tensor | None, eps: float,
+                     out_dtype: torch.dtype) -> torch.Tensor | None:
+    """Layer-scaled residual update fused with the next norm:
+    h (fp32, in place) += s1*a (+ s2*b); returns rms(h)*wn or None."""
+    d = s1.float() * a.float()
+    if b is not None:
+        d = d + s2.float() * b.float()
+    h.add_(d)
+    if wn is None:
+        return None
+    return rmsnorm_rows(h, wn, eps, out_dtype)
+
+
+def xielu(z: torch.Tensor, pq: torch.Tensor) -> torch.Tensor:
+    """Two-parameter squared/exponential unit:
+    z>0: softplus(p) z^2 + z/2;  z<=0: (1/2+softplus(q)) (e^z-1-z) + z/2."""
+    zf = z.float()
+    ap = torch.nn.functional.softplus(pq[0].float())
+    an = 0.5 + torch.nn.functional.softplus(pq[1].float())
+    pos = ap * zf * zf + 0.5 * zf
+    neg = an * (torch.expm1(zf.clamp(max=0.0)) - zf) + 0.5 * zf
+    return torch.where(zf > 0, pos, neg).to(z.dtype)
+
+
+def _row_index(B: int, T: int, pos, lens, slots, device):
+    p = pos.to(torch.int64)
+    ln = (lens.to(torch.int64) if lens is not None
+          else torch.full((B,), T, dtype=torch.int64, device=device))
+    sl = (slots.to(torch.int64) if slots is not None
+          else torch.arange(B, device=device))
+    return p, ln, sl
+
+
+def qknorm_append(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor,
+                  eps: float, nq: int, nkv: int, d: int, dv: int,
+                  kcache: torch.Tensor, vcache: torch.Tensor,
+                  pos: torch.Tensor, T: int, lens=None, slots=None,
+                  per_head: bool = False) -> torch.Tensor:
+    """RMS-normalize q and k (over the whole projection, or per head) and
+    append k, v to the cache. qkv [B*T, nq*d + nkv*d + nkv*dv]; token (b,t)
+    sits at position pos[b]+t of cache row slots[b]; tokens t >= lens[b]
+    are padding (not appended). Returns the normalized q [B*T, nq*d]."""
+    M = qkv.shape[0]
+    B = M // T
+    q = qkv[:, :nq * d]
+    k = qkv[:, nq * d:(nq + nkv) * d]
+    v = qkv[:, (nq + nkv) * d:]
+    if per_head:
+        qn = rmsnorm_rows(q.reshape(M, nq, d), qw, eps, qkv.dtype).reshape(M, -1)
+        kn = rmsnorm_rows(k.reshape(M, nkv, d), kw, eps, qkv.dtype).reshape(M, -1)
+    else:
+        qn = rmsnorm_rows(q, qw, eps, qkv.dtype)
+        kn = rmsnorm_rows(k, kw, eps, qkv.dtype)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, qkv.device)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        kcache[s, :, p0:p0 + n] = kn[b * T:b * T + n].view(n, nkv, d) \
+            .transpose(0, 1).to(kcache.dtype)
+        vcache[s, :, p0:p0 + n] = v[b * T:b * T + n].reshape(n, nkv, dv) \
+            .transpose(0, 1).to(vcache.dtype)
+    return qn
+
+
+def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+             pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
+             temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
+             sinks=None, window: int = 0) -> torch.Tensor:
+    """Causal attention against the cache with score modifiers, all in
+    fp32: s = q.k * scale * temp[h]; s = cap*tanh(s/cap);
+    s -= r1[h] * ln(1 + r2[h] * (i-j)); softmax whose denominator also
+    holds exp(sink[h]). q [B*T, Hq*D] -> out [B*T, Hq*Dv]; query (b,t) is
+    at position pos[b]+t and sees keys j <= that (and > that - window)."""
+    Hkv, D = kcache.shape[1], kcache.shape[3]
+    Dv = vcache.shape[3]
+    M = q.shape[0]
+    B = M // T
+    Hq = q.shape[1] // D
+    G = Hq // Hkv
+    out = torch.zeros(M, Hq * Dv, dtype=q.dtype, device=q.device)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, q.device)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        S = p0 + n
+        kk = kcache[s, :, :S].float()                 # [Hkv, S, D]
+        vv = vcache[s, :, :S].float()
+        qq = q[b * T:b * T + n].float().view(n, Hkv, G, D)
+        sc = torch.einsum("thgd,hsd->hgts", qq, kk) * scale
+        if temp is not None:
+            sc = sc * temp.float().view(Hkv, G, 1, 1)
+        if softcap and softcap > 0:
+            sc = softcap * torch.tanh(sc / softcap)
+        i = torch.arange(p0, S, device=q.device).view(n, 1)
+        j = torch.arange(S, device=q.device).view(1, S)
+        dist = (i - j)
+        if dist_r1 is not None:
+            sc = sc - dist_r1.float().view(Hkv, G, 1, 1) * torch.log1p(
+                dist_r2.float().view(Hkv, G, 1, 1)
+                * dist.clamp(min=0).float())
+        dead = dist < 0
+        if window and window > 0:
+            dead = dead | (dist >= window)
+        sc = sc.masked_fill(dead, float("-inf"))
+        if sinks is not None:
+            sk = sinks.float().view(Hkv, G, 1, 1).expand(Hkv, G, n, 1)
+            pr = torch.softmax(torch.cat([sc, sk], dim=-1), dim=-1)[..., :-1]
+        else:
+            pr = torch.softmax(sc, dim=-1)
+        o = torch.einsum("hgts,hsd->thgd", pr, vv)
+        out[b * T:b * T + n] = o.reshape(n, Hq * Dv).to(q.dtype)
+    return out

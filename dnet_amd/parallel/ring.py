@@ -134,14 +134,17 @@ class RingExecutor:
         self.sampler = Sampler(decoding or DecodingConfig())
         H = cfg.hidden_size
         # static buffers (recv targets / graph inputs)
-        self.hbuf = [torch.zeros(mb_size, H, dtype=torch.bfloat16,
+        # (residual-stream dtype is the model's: bf16, or fp32 for
+        # families that keep the residual in 32-bit)
+        self.hbuf = [torch.zeros(mb_size, H, dtype=self.model.act_dtype,
                                  device=self.device) for _ in range(mb_count)]
         self.tokbuf = [torch.zeros(mb_size, dtype=torch.int64,
                                    device=self.device) for _ in range(mb_count)]
         self.logits_buf = None
         if self.is_last:
             self.logits_buf = [torch.zeros(mb_size, cfg.vocab_size,
-                                           dtype=torch.bfloat16, device=self.device)
+                                           dtype=self.model.logits_dtype,
+                                           device=self.device)
                                for _ in range(mb_count)]
         if use_graphs is None:
             use_graphs = self.device.type == "cuda"
@@ -217,8 +220,7 @@ class RingExecutor:
 
     def _decode_body(self, mb: int, r: int = 0):
         if self.is_first and r == 0:
-            self.hbuf[mb].copy_(
-                torch.nn.functional.embedding(self.tokbuf[mb], self.model.embed))
+            self.hbuf[mb].copy_(self.model.embed_tokens(self.tokbuf[mb]))
         if self.windows[r]:
             self.model.decode_window(self.hbuf[mb], self.windows[r],
                                      self.kvs[mb])
@@ -305,7 +307,7 @@ class RingExecutor:
                     else:
                         if h is None:
                             h = torch.empty(B, p1 - p0, H,
-                                            dtype=torch.bfloat16,
+                                            dtype=self.model.act_dtype,
                                             device=self.device)
                         self.ring.recv(h)
                     if self.windows[r]:
@@ -437,33 +439,127 @@ class RingExecutor:
         other slots keep decoding state. ``tokens`` [T] int64 (significant
         on the first stage). Returns the last-position logits [1, V] on
         the LAST stage, else None."""
-        T = int(tokens.shape[-1])
+        out = self.prefill_slots([si], [tokens.view(-1)], chunk=chunk)
+        return out[0] if out is not None else None
+
+    def prefill_slots(self, slots: list, prompts: list, want=None,
+                      chunk: int = 2048, start=None):
+        """Collective prefill of several prompts of unequal length into the
+        KV slots ``slots`` while other slots keep their state. Models with
+        ``ragged_prefill`` take the whole batch in one pass (rows
+        right-padded to the longest prompt, per-row lengths on the device);
+        the others go slot by slot. ``want[i]``: positions of prompt i
+        whose logits are returned (default: its last). ``start[i]``: tokens
+        slot i already holds (default 0: a fresh request); the prompt then
+        continues from there. Position-chunked by ``chunk`` to bound
+        activations. Returns a list of logits
+        [len(want[i]), V] on the LAST stage, else None."""
+        n = len(slots)
+        lens = [int(p.shape[-1]) for p in prompts]
+        if want is None:
+            want = [[t - 1] for t in lens]
+        if start is None:
+            start = [0] * n
+        assert max(s + t for s, t in zip(start, lens)) <= self.smax, \
+            "prompt longer than the KV capacity"
+        groups = ([list(range(n))] if self.model.ragged_prefill
+                  else [[i] for i in range(n)])
         H = self.cfg.hidden_size
-        kvslot = self.kvs[0].slot(si)
-        kvslot.pos.fill_(0)
-        step = chunk if 0 < chunk < T else T
-        h = None
-        for p0 in range(0, T, step):
-            p1 = min(p0 + step, T)
-            h = None
-            for r in range(self.rounds):
-                if self.is_first and r == 0:
-                    h = self.model.embed_tokens(
-                        tokens.view(1, T)[:, p0:p1].to(self.device)).clone()
-                else:
-                    if h is None:
-                        h = torch.empty(1, p1 - p0, H, dtype=torch.bfloat16,
-                                        device=self.device)
-                    self.ring.recv(h)
-                if self.windows[r]:
-                    self.model.prefill_window(h, self.windows[r], kvslot, p0)
-                if not (self.is_last and r == self.rounds - 1):
-                    if self.stages > 1:
-                        self.ring.send(h)
-        kvslot.pos.fill_(T)
-        if self.is_last:
-            return self.model.normalize_project(h[:, -1].contiguous())
-        return None
+        kv = self.kvs[0]
+        picked: list = [[] for _ in range(n)]
+        for grp in groups:
+            Tm = max(lens[i] for i in grp)
+            step = chunk if 0 < chunk < Tm else Tm
+            B = len(grp)
+            if self.model.ragged_prefill:
+                tok = torch.zeros(B, Tm, dtype=torch.int64)
+                for r, i in enumerate(grp):
+                    tok[r, :lens[i]] = prompts[i].view(-1).cpu()
+                slot_t = torch.tensor([slots[i] for i in grp],
+                                      dtype=torch.int32, device=self.device)
+                len_t = torch.tensor([lens[i] for i in grp],
+                                     dtype=torch.int32, device=self.device)
+                start_t = torch.tensor([start[i] for i in grp],
+                                       dtype=torch.int32, device=self.device)
+            else:
+                tok = prompts[grp[0]].view(1, Tm)
+                kvslot = kv.slot(slots[grp[0]])
+                kvslot.pos.fill_(start[grp[0]])
+            for p0 in range(0, Tm, step):
+                p1 = min(p0 + step, Tm)
+                h = None
+                for r in range(self.rounds):
+                    if self.is_first and r == 0:
+                        h = self.model.embed_tokens(
+                            tok[:, p0:p1].to(self.device)).clone()
+                    else:
+                        if h is None:
+                            h = torch.empty(B, p1 - p0, H,
+                                            dtype=self.model.act_dtype,
+                                            device=self.device)
+                        self.ring.recv(h)
+                    if self.windows[r]:
+                        if self.model.ragged_prefill:
+                            self.model.prefill_window(
+                                h, self.windows[r], kv, start_t + p0,
+                                lens=(len_t - p0).clamp_(0, p1 - p0),
+                                slots=slot_t)
+                        else:
+                            self.model.prefill_window(
+                                h, self.windows[r], kvslot,
+                                start[grp[0]] + p0)
+                    if not (self.is_last and r == self.rounds - 1):
+                        if self.stages > 1:
+                            self.ring.send(h)
+                if self.is_last:
+                    for r_, i in enumerate(grp):
+                        for w in want[i]:
+                            if p0 <= w < p1:
+                                picked[i].append(h[r_, w - p0])
+            for i in grp:
+                kv.pos[slots[i]] = start[i] + lens[i]
+        if not self.is_last:
+            return None
+        rows = [r for p in picked for r in p]
+        if not rows:
+            return [None] * n
+        logits = self.model.normalize_project(torch.stack(rows).contiguous())
+        out, at = [], 0
+        for i in range(n):
+            out.append(logits[at:at + len(picked[i])])
+            at += len(picked[i])
+        return out
+
+    def slot_advance(self, park: torch.Tensor, free: torch.Tensor) -> None:
+        """After a slot-batch decode step: every row moves one position on;
+        parked rows (bool mask ``park``: free or mid-prefill slots) are
+        pinned at the last cache row so their dummy append stays in range,
+        and ``free`` rows at position 0 so a dead row scans one key. Device
+        ops only."""
+        pos = self.kvs[0].pos
+        pos.add_(1)
+        pos.masked_fill_(park, self.smax - 1)
+        pos.masked_fill_(free, 0)
+
+    def resize_slots(self, n: int) -> None:
+        """Grow the slot batch to ``n`` rows (live slots keep their cache);
+        captured decode graphs are dropped and re-captured on next use."""
+        if n <= self.mb_size:
+            return
+        assert self.mb_count == 1
+        self.kvs[0].grow(n)
+        self.hbuf = [torch.zeros(n, self.cfg.hidden_size,
+                                 dtype=self.model.act_dtype,
+                                 device=self.device)]
+        tb = torch.zeros(n, dtype=torch.int64, device=self.device)
+        tb[:self.mb_size] = self.tokbuf[0]
+        self.tokbuf = [tb]
+        if self.logits_buf is not None:
+            self.logits_buf = [torch.zeros(n, self.cfg.vocab_size,
+                                           dtype=self.model.logits_dtype,
+                                           device=self.device)]
+        self.mb_size = n
+        self._graphs = {}
 
     t_replay = 0.0   # cumulative; slot-tick profiling
 

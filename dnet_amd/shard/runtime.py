@@ -124,12 +124,21 @@ class ShardRuntime:
             group = int(req.quant.split("-g")[1]) if "-g" in req.quant else 128
             quant = QuantConfig(bits, group)
         p = Path(req.model_path).expanduser()
-        if (p / "config.json").exists():
-            return ModelConfig.from_hf(json.loads((p / "config.json").read_text()),
-                                       quant=quant)
         name = req.model_name or req.model_path
-        if name in PRESETS:
-            return ModelConfig.from_hf(dict(PRESETS[name]), quant=quant)
+        cfg = None
+        if (p / "config.json").exists():
+            cfg = ModelConfig.from_hf(
+                json.loads((p / "config.json").read_text()), quant=quant)
+        elif name in PRESETS:
+            cfg = ModelConfig.from_hf(dict(PRESETS[name]), quant=quant)
+        if cfg is not None:
+            if req.dtype == "float32":
+                from ..models import get_ring_model
+                if not getattr(get_ring_model(cfg.model_type),
+                               "supports_float32", False):
+                    raise ValueError(f"{cfg.model_type}: no float32 path")
+            cfg.compute_dtype = req.dtype
+            return cfg
         raise FileNotFoundError(
             f"model not found: {req.model_path!r} (no config.json, not a preset)")
 
@@ -755,9 +764,7 @@ class ShardRuntime:
         if ex.world > 1:
             import torch.distributed as dist
             dist.broadcast(ex.tokbuf[0], src=(ex.stages - 1) * ex.tp)
-        ex.kvs[0].pos.add_(1)
-        ex.kvs[0].pos.masked_fill_(self._park_dev, ex.smax - 1)
-        ex.kvs[0].pos.masked_fill_(self._free_dev, 0)
+        ex.slot_advance(self._park_dev, self._free_dev)
         self._slot_emit(ex.tokbuf[0],
                         [(i, self._slot_gen[i])
                          for i, st in enumerate(self.slots)
@@ -791,15 +798,13 @@ class ShardRuntime:
         self._t_sample += time.perf_counter() - t0
         t0 = time.perf_counter()
         ex.tokbuf[0].copy_(toks_t)
-        ex.kvs[0].pos.add_(1)
         # park idle/prefilling slots at the last row: the dummy append
         # stays in range and that row is rewritten by a real token before
         # any active slot ever attends to it. Device-resident mask:
         # building a park index tensor here was a synchronous H2D that
         # serialized the host against the in-flight decode graph
         # (~17 ms/tick measured).
-        ex.kvs[0].pos.masked_fill_(self._park_dev, ex.smax - 1)
-        ex.kvs[0].pos.masked_fill_(self._free_dev, 0)
+        ex.slot_advance(self._park_dev, self._free_dev)
         if self._launch_evs is not None:
             self._launch_evs[1].record()
         self._t_aux += time.perf_counter() - t0

@@ -15,7 +15,8 @@ from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Iterator, Optional
 
-_LAYER_RE = re.compile(r"^(?:model\.)?layers\.(\d+)\.(.+)$")
+# "layers.N." (HF layouts) or "lN." (posudra layout)
+_LAYER_RE = re.compile(r"^(?:model\.)?(?:layers\.|l)(\d+)\.(.+)$")
 _DTYPE_BYTES = {"F64": 8, "F32": 4, "F16": 2, "BF16": 2, "I64": 8, "I32": 4,
                 "I16": 2, "I8": 1, "U8": 1, "BOOL": 1, "F8_E4M3": 1,
                 "F8_E5M2": 1}
@@ -79,11 +80,12 @@ def get_model_metadata(model_dir: str) -> ModelMetadata:
             m = _LAYER_RE.match(ti.name)
             if m:
                 meta.layers.setdefault(int(m.group(1)), []).append(ti.name)
-            elif "embed_tokens" in ti.name:
+            elif "embed_tokens" in ti.name or ti.name == "embed":
                 meta.embed.append(ti.name)
-            elif "lm_head" in ti.name:
+            elif "lm_head" in ti.name or ti.name == "head":
                 meta.lm_head.append(ti.name)
-            elif ti.name in ("model.norm.weight", "norm.weight"):
+            elif ti.name in ("model.norm.weight", "norm.weight",
+                             "final.norm"):
                 meta.final_norm.append(ti.name)
             else:
                 meta.other.append(ti.name)
