@@ -64,6 +64,28 @@ void moe_down(torch::Tensor act, torch::Tensor w,
 void col_norm2(torch::Tensor x, torch::Tensor norms);
 void gather_cols(torch::Tensor x, torch::Tensor idx, torch::Tensor out);
 void scatter_cols(torch::Tensor in, torch::Tensor idx, torch::Tensor out);
+void rmsnorm_rows(torch::Tensor x, torch::Tensor w, torch::Tensor y,
+                  double eps);
+void ls_resid_rmsnorm(torch::Tensor h, torch::Tensor a, torch::Tensor s1,
+                      c10::optional<torch::Tensor> b,
+                      c10::optional<torch::Tensor> s2,
+                      c10::optional<torch::Tensor> wn,
+                      c10::optional<torch::Tensor> y, double eps);
+void xielu(torch::Tensor z, torch::Tensor pq, torch::Tensor y);
+void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
+                   torch::Tensor qout, torch::Tensor kcache,
+                   torch::Tensor vcache, torch::Tensor pos,
+                   c10::optional<torch::Tensor> lens,
+                   c10::optional<torch::Tensor> slots, double eps, int64_t nq,
+                   int64_t nkv, int64_t d, int64_t dv, int64_t T,
+                   bool per_head);
+void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
+              torch::Tensor pos, c10::optional<torch::Tensor> lens,
+              c10::optional<torch::Tensor> slots, torch::Tensor out,
+              int64_t T, double scale, c10::optional<torch::Tensor> temp,
+              double softcap, c10::optional<torch::Tensor> dist_r1,
+              c10::optional<torch::Tensor> dist_r2,
+              c10::optional<torch::Tensor> sinks, int64_t window);
 }  // namespace dnet
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -115,4 +137,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("col_norm2", &dnet::col_norm2, "per-column L2 norms");
   m.def("gather_cols", &dnet::gather_cols, "pack kept columns");
   m.def("scatter_cols", &dnet::scatter_cols, "zero + scatter kept columns");
+  m.def("rmsnorm_rows", &dnet::rmsnorm_rows,
+        "RMSNorm with fp32 statistics, fp32/bf16 in and out");
+  m.def("ls_resid_rmsnorm", &dnet::ls_resid_rmsnorm,
+        "fp32 residual += layer-scaled branches, fused with the next norm");
+  m.def("xielu", &dnet::xielu, "two-parameter squared/exponential unit");
+  m.def("qknorm_append", &dnet::qknorm_append,
+        "q/k RMSNorm (whole projection or per head) + KV append");
+  m.def("attn_mod", &dnet::attn_mod,
+        "score-modified causal attention (decode + ragged prefill)");
 }
