@@ -466,7 +466,7 @@ class RingExecutor:
                   else [[i] for i in range(n)])
         H = self.cfg.hidden_size
         kv = self.kvs[0]
-        picked: list = [[] for _ in range(n)]
+        picked: list = [[None] * len(w) for w in want]
         for grp in groups:
             Tm = max(lens[i] for i in grp)
             step = chunk if 0 < chunk < Tm else Tm
@@ -513,9 +513,9 @@ class RingExecutor:
                             self.ring.send(h)
                 if self.is_last:
                     for r_, i in enumerate(grp):
-                        for w in want[i]:
+                        for k, w in enumerate(want[i]):
                             if p0 <= w < p1:
-                                picked[i].append(h[r_, w - p0])
+                                picked[i][k] = h[r_, w - p0]
             for i in grp:
                 kv.pos[slots[i]] = start[i] + lens[i]
         if not self.is_last:

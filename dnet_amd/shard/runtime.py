@@ -523,8 +523,14 @@ class ShardRuntime:
         active = any(s is not None for s in self.slots)
         block = not active
         progressed = False
-        while any(s is None for s in self.slots):
-            free = next(i for i, s in enumerate(self.slots) if s is None)
+        chunk = int(os.environ.get("DNET_PREFILL_CHUNK", "2048"))
+        ragged = ex.world == 1 and ex.model.ragged_prefill
+        batch: list = []            # (slot, frame) admitted in one prefill
+        taken: set = set()
+        while any(s is None and i not in taken
+                  for i, s in enumerate(self.slots)):
+            free = next(i for i, s in enumerate(self.slots)
+                        if s is None and i not in taken)
             try:
                 frame = (self.infer_q.get(timeout=0.02) if block
                          else self.infer_q.get_nowait())
@@ -532,11 +538,22 @@ class ShardRuntime:
                 break
             block = False
             progressed = True
+            if ragged and int(frame.get("prompt_len", chunk + 1)) <= chunk:
+                batch.append((free, frame))
+                taken.add(free)
+                continue
             try:
                 self._slot_admit(free, frame)
             except Exception:
                 log.exception("slot admit failed")
                 self._send_error(frame.get("nonce", ""))
+        if batch:
+            try:
+                self._slot_admit_batch(batch)
+            except Exception:
+                log.exception("slot batch admit failed")
+                for _, frame in batch:
+                    self._send_error(frame.get("nonce", ""))
         prefilling = [i for i, st in enumerate(self.slots)
                       if st is not None and st.get("state") == "prefill"]
         if prefilling:
@@ -682,6 +699,15 @@ class ShardRuntime:
                      "(chunked)", si, nonce[:18], int(tokens.shape[-1]))
             return
         logits = ex.prefill_slot(si, tokens)
+        self._slot_admit_finish(si, logits, int(tokens.shape[-1]), max_tokens,
+                                stop_ids, nonce, cfg, gen)
+
+    def _slot_admit_finish(self, si, logits, T, max_tokens, stop_ids, nonce,
+                           cfg, gen) -> None:
+        """Second half of an admit: sample the first token from the
+        prefill's last-position logits, broadcast it, emit it and register
+        the slot."""
+        ex = self.executor
         t0_t = torch.zeros(1, dtype=torch.int64, device=self._comm_device())
         lp0 = tops0 = None
         if ex.is_last:
@@ -707,7 +733,38 @@ class ShardRuntime:
             self._park_dev[si] = False
             self._free_dev[si] = False
         log.info("[PROFILE][SLOT] admit slot=%d nonce=%s prompt=%d", si,
-                 nonce[:18], int(tokens.shape[-1]))
+                 nonce[:18], T)
+
+    def _slot_admit_batch(self, items: list) -> None:
+        """Admit several queued requests in ONE ragged prefill (models with
+        ``ragged_prefill``, single rank): prompts of unequal length share
+        the pass, each landing in its own KV slot. ``items``: (slot, frame)
+        pairs."""
+        import numpy as np
+        ex = self.executor
+        metas, slots, prompts = [], [], []
+        for si, frame in items:
+            tokens = torch.from_numpy(np.frombuffer(
+                frame["tokens"], dtype=np.int32).copy()).long().view(-1)
+            p = frame.get("params", {})
+            cfg = DecodingConfig(
+                temperature=p.get("temperature", 0.0),
+                top_p=p.get("top_p", 1.0), top_k=int(p.get("top_k", 0)),
+                min_p=p.get("min_p", 0.0),
+                logprobs=bool(p.get("logprobs", False)),
+                top_logprobs=int(p.get("top_logprobs", 0)))
+            self._slot_gen[si] += 1
+            T = int(tokens.shape[-1])
+            max_tokens = max(1, min(int(frame.get("max_tokens", 128)),
+                                    ex.smax - T))
+            gen = self._row_sampler.set_row(si, cfg, p.get("seed"))
+            metas.append((si, T, max_tokens, list(frame.get("stop_ids", [])),
+                          frame.get("nonce", ""), cfg, gen))
+            slots.append(si)
+            prompts.append(tokens)
+        logits = ex.prefill_slots(slots, prompts)
+        for m, lg in zip(metas, logits):
+            self._slot_admit_finish(m[0], lg, *m[1:])
 
     def _slot_prefill_chunk(self, si: int) -> None:
         """Feed one position chunk of a prefilling slot's prompt; on the
