@@ -47,6 +47,79 @@ from dnet_amd.parallel.comm import init_from_env
 from dnet_amd.parallel.ring import RingExecutor
 
 
+# equal-size family comparison: (name, width, heads, kv_heads, head_dim, ff)
+_COMPARE_SIZES = [("2k", 2048, 16, 4, 128, 8192),
+                  ("4k", 4096, 32, 8, 128, 12288),
+                  ("5k", 5120, 64, 8, 128, 25600)]
+
+
+def compare_posudra(args, device):
+    """Prefill and decode throughput of posudra beside the closest existing
+    family (qwen3: dense, grouped heads, q/k norm) at equal layer sizes,
+    bf16, random weights. One JSON line; the default workload is untouched."""
+    from dnet_amd.models.config import posudra_config
+    layers, vocab = args.compare_layers, 32768
+    B, T, Bd = args.compare_prefill_batch, args.prompt_len, args.mb_size
+    rows = []
+    for name, W, H, KV, D, FF in _COMPARE_SIZES:
+        if args.compare_sizes and name not in args.compare_sizes.split(","):
+            continue
+        row = {"size": name, "width": W, "heads": H, "kv_heads": KV,
+               "head_dim": D, "ff": FF, "layers": layers}
+        for fam in ("posudra", "qwen3"):
+            if fam == "posudra":
+                hf = posudra_config(W, layers, H, KV, D, D, FF, vocab)
+            else:
+                hf = dict(model_type="qwen3", hidden_size=W,
+                          num_hidden_layers=layers, num_attention_heads=H,
+                          num_key_value_heads=KV, head_dim=D,
+                          intermediate_size=FF, vocab_size=vocab,
+                          rope_theta=1000000.0, rms_norm_eps=1e-6)
+            cfg = ModelConfig.from_hf(hf)
+            g = torch.Generator().manual_seed(7)
+            # prefill: B prompts of T tokens, eager (as serving runs it)
+            ex = RingExecutor(cfg, 0, 1, device, mb_count=1, mb_size=B,
+                              smax=args.smax, seed=1234, use_graphs=False)
+            toks = torch.randint(0, vocab, (1, B, T), generator=g).to(device)
+            ts = []
+            for _ in range(4):
+                ex.reset()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                ex.prefill(toks)
+                torch.cuda.synchronize()
+                ts.append(time.perf_counter() - t0)
+            row[fam + "_prefill_tok_s"] = round(B * T / min(ts[1:]), 1)
+            del ex
+            torch.cuda.empty_cache()
+            # decode: Bd sequences at context ~T, hipGraph steps
+            ex = RingExecutor(cfg, 0, 1, device, mb_count=1, mb_size=Bd,
+                              smax=args.smax, seed=1234,
+                              use_graphs=not args.no_graphs)
+            toks = torch.randint(0, vocab, (1, Bd, T), generator=g).to(device)
+            ex.prefill(toks)
+            ex.decode_rounds(args.warmup, collect=False)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ex.decode_rounds(args.steps, collect=False)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            row[fam + "_decode_tok_s"] = round(Bd * args.steps / dt, 1)
+            row[fam + "_decode_ms_step"] = round(dt / args.steps * 1e3, 3)
+            del ex
+            torch.cuda.empty_cache()
+        rows.append(row)
+    print(json.dumps({
+        "metric": "posudra vs qwen3 at equal layer sizes: prefill and "
+                  "decode tokens/s (1 GPU, bf16)",
+        "dtype": "bf16", "data": "synthetic (random tokens, random-init "
+                                 "weights)",
+        "prefill": {"batch": B, "prompt_len": T},
+        "decode": {"batch": Bd, "context": T, "steps": args.steps,
+                   "warmup": args.warmup},
+        "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -76,10 +149,28 @@ def main():
     ap.add_argument("--residency", type=int, default=0,
                     help="GPU-resident layers per rank (0=all; <local layers "
                          "enables host-DRAM weight streaming)")
+    ap.add_argument("--compare-family", default="", choices=["", "posudra"],
+                    help="instead of the default workload: throughput of "
+                         "this family beside its closest existing one at "
+                         "equal layer sizes")
+    ap.add_argument("--compare-layers", type=int, default=8)
+    ap.add_argument("--compare-prefill-batch", type=int, default=8)
+    ap.add_argument("--compare-sizes", default="",
+                    help="comma list out of 2k,4k,5k (default: all)")
     args = ap.parse_args()
 
     rank, world, device = init_from_env()
     on_gpu = device.type == "cuda"
+    if args.compare_family:
+        assert world == 1 and on_gpu, "family comparison: one GPU"
+        if args.prompt_len == 128:
+            args.prompt_len = 1024
+        args.smax = max(args.smax, args.prompt_len + args.steps
+                        + args.warmup + 64)
+        if args.mb_size == 64:
+            args.mb_size = 32
+        compare_posudra(args, device)
+        return
 
     quant = None
     if args.quant == "int8":

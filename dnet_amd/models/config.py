@@ -173,6 +173,21 @@ class ModelConfig:
         return mc
 
 
+def posudra_config(width: int, layers: int, heads: int, kv_heads: int,
+                   dim: int, vdim: int, ff: int, vocab: int,
+                   softcap: float = 50.0, eps: float = 1e-5,
+                   embedding_scale: float = 1.0) -> dict:
+    """A uniform posudra stack in the checkpoint's config.json layout."""
+    layer = {"type": "attention",
+             "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim,
+                       "vdim": vdim, "scale": dim ** -0.5,
+                       "softcap": softcap},
+             "mlp": {"kind": "dense", "ff": ff} if ff else None}
+    return {"architecture": "Posudra", "vocab": vocab, "width": width,
+            "norm": {"eps": eps}, "embedding": {"scale": embedding_scale},
+            "layers": [dict(layer) for _ in range(layers)]}
+
+
 # Known configs for synthetic benchmarking (random-init weights; no network).
 PRESETS: dict[str, dict] = {
     "llama-3-8b": dict(model_type="llama", hidden_size=4096, num_hidden_layers=32,
@@ -230,6 +245,11 @@ PRESETS: dict[str, dict] = {
                              topk_group=4, scoring_func="sigmoid",
                              norm_topk_prob=True,
                              routed_scaling_factor=2.5, rope_theta=10000.0),
+    # posudra at qwen3-8b's layer sizes (equal-size family comparison)
+    "posudra-8b-like": posudra_config(4096, 36, 32, 8, 128, 128, 12288,
+                                      151936),
+    "posudra-tiny": posudra_config(128, 4, 4, 2, 32, 16, 192, 256,
+                                   softcap=8.0, embedding_scale=4.0),
     "tiny": dict(model_type="llama", hidden_size=128, num_hidden_layers=4,
                  num_attention_heads=2, num_key_value_heads=2, head_dim=64,
                  intermediate_size=256, vocab_size=256, rope_theta=10000.0),

@@ -133,17 +133,21 @@ class PosudraRingModel(RingModel):
         c = self.cfg
         W = c.hidden_size
 
+        on_gpu = self.device.type == "cuda"
+        gdev = self.device if on_gpu else "cpu"
+
         def gen(sub):
-            g = torch.Generator()
+            g = torch.Generator(device=gdev)
             g.manual_seed(seed * 100003 + sub)
             return g
 
         def rn(g, *shape, std=1.0):
-            return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16)
+            return (torch.randn(*shape, generator=g, device=gdev)
+                    * std).to(torch.bfloat16)
 
         def ru(g, n, lo, hi):
-            return (torch.rand(n, generator=g) * (hi - lo) + lo).to(
-                torch.bfloat16)
+            return (torch.rand(n, generator=g, device=gdev)
+                    * (hi - lo) + lo).to(torch.bfloat16)
 
         for lid in self.layer_ids:
             g = gen(lid)

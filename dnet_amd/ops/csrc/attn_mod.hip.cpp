@@ -226,6 +226,182 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
   }
 }
 
+// ---- bf16 prefill on the matrix cores -------------------------------------
+// Block = 4 waves, each owning 16 query tokens of a 64-token tile of one
+// head (grid = token tiles x Hq x batch rows). Per 32-key tile the waves
+// stage K [32][DC*32] and V transposed [NV*16][32] in LDS (head sizes
+// zero-padded), QK^T = 2 x DC MFMAs into fp32 C fragments (lane holds
+// q = hi*4+r, key = lane&15), modifiers + online softmax on the fragments,
+// P relayed through a per-wave LDS slab as the A operand of NV PV MFMAs.
+__device__ __forceinline__ float fast_tanh(float x) {
+  // 1 - 2/(e^{2x}+1): saturates cleanly (e^{2x} -> inf or 0)
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f);
+}
+
+template <int DC, int NV>
+__global__ __launch_bounds__(256) void attn_mod_mfma(
+    const short* __restrict__ q, const short* __restrict__ kc,
+    const short* __restrict__ vc, short* __restrict__ out,
+    const ModParams P) {
+  constexpr int ST = 32;
+  constexpr int DP = DC * 32, DVP = NV * 16;
+  constexpr int KP = DP + 8, SP = ST + 8;
+  __shared__ short k_lds[ST * KP];
+  __shared__ short vt_lds[DVP * SP];
+  __shared__ short p_lds[4][16 * SP];
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int hk = h / (P.Hq / P.Hkv);
+  const int D = P.D, DV = P.DV;
+  const int n = P.lens ? min(P.lens[b], P.T) : P.T;
+  const int tile0 = blockIdx.x * 64;
+  if (tile0 >= n) return;
+  const int slot = P.slots ? P.slots[b] : b;
+  if (slot < 0 || slot >= P.Bc) return;
+  const int p0 = P.pos[b];
+  const int qt = tile0 + wave * 16;
+  const int row = lane & 15, hi = lane >> 4;
+  const int qrow = min(qt + row, n - 1);
+  const short* qp = q + ((int64_t)b * P.T + qrow) * P.Hq * D + (int64_t)h * D;
+  const short* kp = kc + ((int64_t)slot * P.Hkv + hk) * P.Smax * D;
+  const short* vp = vc + ((int64_t)slot * P.Hkv + hk) * P.Smax * DV;
+
+  bf16x8 qf[DC];
+#pragma unroll
+  for (int c = 0; c < DC; ++c) {
+    const int e0 = c * 32 + hi * 8;
+    short8 z;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) z.x[j] = 0;
+    if (e0 < D) z = *reinterpret_cast<const short8*>(&qp[e0]);
+    qf[c] = *reinterpret_cast<const bf16x8*>(&z);
+  }
+  f32x4 acc[NV];
+#pragma unroll
+  for (int nn = 0; nn < NV; ++nn) acc[nn] = {0.f, 0.f, 0.f, 0.f};
+  float m_run[4], l_run[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    m_run[r] = -1e30f;
+    l_run[r] = 0.f;
+  }
+  const float sc_t = P.scale * (P.temp ? P.temp[h] : 1.f);
+  const float cap = P.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+  const float r1 = P.r1 ? P.r1[h] : 0.f, r2 = P.r1 ? P.r2[h] : 0.f;
+
+  const int q_hi = min(tile0 + 63, n - 1);
+  const int s_end = min(P.Smax, p0 + q_hi + 1);
+  int s_begin = 0;
+  if (P.window > 0) s_begin = max(0, p0 + tile0 - P.window + 1) & ~(ST - 1);
+
+  for (int s0 = s_begin; s0 < s_end; s0 += ST) {
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < ST * (DP / 8); idx += 256) {
+      const int sr = idx / (DP / 8), dc = (idx % (DP / 8)) * 8;
+      const int sg = min(s0 + sr, P.Smax - 1);
+      short8 z;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) z.x[j] = 0;
+      if (dc < D) z = *reinterpret_cast<const short8*>(&kp[(int64_t)sg * D + dc]);
+      *reinterpret_cast<short8*>(&k_lds[sr * KP + dc]) = z;
+    }
+    for (int idx = threadIdx.x; idx < ST * (DVP / 2); idx += 256) {
+      const int sr = idx / (DVP / 2), dc = (idx % (DVP / 2)) * 2;
+      const int sg = min(s0 + sr, P.Smax - 1);
+      short v0 = 0, v1 = 0;
+      if (dc < DV) {              // DV is even (multiple of 8)
+        v0 = vp[(int64_t)sg * DV + dc];
+        v1 = vp[(int64_t)sg * DV + dc + 1];
+      }
+      vt_lds[dc * SP + sr] = v0;
+      vt_lds[(dc + 1) * SP + sr] = v1;
+    }
+    __syncthreads();
+
+    float p_val[2][4], m_new[4];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
+            &k_lds[(sub * 16 + row) * KP + c * 32 + hi * 8]);
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c], kf, sc, 0, 0, 0);
+      }
+      const int j = s0 + sub * 16 + row;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int qq = qt + hi * 4 + r;
+        const int i = p0 + qq;
+        float val = sc[r] * sc_t;
+        if (cap > 0.f) val = cap * fast_tanh(val * inv_cap);
+        if (P.r1) val -= r1 * __logf(1.f + r2 * (float)max(i - j, 0));
+        bool dead = (j > i) || (qq >= n) || (j >= P.Smax);
+        if (P.window > 0) dead |= (j <= i - P.window);
+        p_val[sub][r] = dead ? -INFINITY : val;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float mx = fmaxf(p_val[0][r], p_val[1][r]);
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1)
+        mx = fmaxf(mx, __shfl_xor(mx, off, 16));
+      m_new[r] = fmaxf(m_run[r], mx);
+      const float corr = __expf(m_run[r] - m_new[r]);
+      float ls = 0.f;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        p_val[sub][r] = __expf(p_val[sub][r] - m_new[r]);
+        ls += p_val[sub][r];
+      }
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) ls += __shfl_xor(ls, off, 16);
+      l_run[r] = l_run[r] * corr + ls;
+      m_run[r] = m_new[r];
+#pragma unroll
+      for (int nn = 0; nn < NV; ++nn) acc[nn][r] *= corr;
+    }
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        p_lds[wave][(hi * 4 + r) * SP + sub * 16 + row] =
+            f2bits(p_val[sub][r]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // wave-local slab
+    const bf16x8 pf =
+        *reinterpret_cast<const bf16x8*>(&p_lds[wave][row * SP + hi * 8]);
+#pragma unroll
+    for (int nn = 0; nn < NV; ++nn) {
+      const bf16x8 vf = *reinterpret_cast<const bf16x8*>(
+          &vt_lds[(nn * 16 + row) * SP + hi * 8]);
+      acc[nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, acc[nn], 0,
+                                                        0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int qq = qt + hi * 4 + r;
+    if (qq >= n) continue;
+    float c = 1.f;
+    if (P.sinks) {
+      const float sk = P.sinks[h];
+      const float m2 = fmaxf(m_run[r], sk);
+      c = __expf(m_run[r] - m2);
+      l_run[r] = l_run[r] * c + __expf(sk - m2);
+    }
+    const float inv = l_run[r] > 0.f ? c / l_run[r] : 0.f;
+    short* op = out + ((int64_t)b * P.T + qq) * P.Hq * DV + (int64_t)h * DV;
+#pragma unroll
+    for (int nn = 0; nn < NV; ++nn) {
+      const int dv = nn * 16 + row;
+      if (dv < DV) op[dv] = f2bits(acc[nn][r] * inv);
+    }
+  }
+}
+
 }  // namespace
 
 static const float* opt_f32(const c10::optional<torch::Tensor>& t, int64_t n,
@@ -296,6 +472,29 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
   DNET_CHECK(lds <= 160 * 1024, "attn_mod: head sizes exceed LDS");
   const dim3 grid((unsigned)((T + P.QT - 1) / P.QT), (unsigned)(Hkv * GS),
                   (unsigned)B);
+  // bf16 prompts: matrix-core kernel (head sizes padded to its tile classes)
+  if (!f32 && T >= 16 && D % 8 == 0 && DV % 8 == 0) {
+    const dim3 mgrid((unsigned)((T + 63) / 64), (unsigned)Hq, (unsigned)B);
+#define AM(DCC, NVV)                                                         \
+  hipLaunchKernelGGL((attn_mod_mfma<DCC, NVV>), mgrid, dim3(256), 0, stream, \
+                     (const short*)q.data_ptr(),                             \
+                     (const short*)kcache.data_ptr(),                        \
+                     (const short*)vcache.data_ptr(), (short*)out.data_ptr(), \
+                     P)
+#define AM_V(DCC)                          \
+  do {                                     \
+    if (DV <= 64) AM(DCC, 4);              \
+    else if (DV <= 128) AM(DCC, 8);        \
+    else AM(DCC, 16);                      \
+  } while (0)
+    if (D <= 64) AM_V(2);
+    else if (D <= 128) AM_V(4);
+    else if (D <= 192) AM_V(6);
+    else AM_V(8);
+#undef AM_V
+#undef AM
+    return;
+  }
   if (f32) {
     if (lds > 64 * 1024)
       DNET_CHECK_HIP(hipFuncSetAttribute(
