@@ -485,6 +485,16 @@ def qknorm_append(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor,
                              vcache, pos, T, lens, slots, per_head)
 
 
+def _attn_mod_splits(blocks: int, smax: int) -> int:
+    """Split-KV factor for the decode kernel: aim at >= ~1024 workgroups
+    (4 per CU) while every split keeps >= 256 positions of cache capacity.
+    A function of static shapes only, so captured graphs stay valid."""
+    splits = 1
+    while blocks * splits < 1024 and splits * 2 * 256 <= smax:
+        splits *= 2
+    return splits
+
+
 def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
              pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
              temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
@@ -497,11 +507,19 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
         Hkv, D = kcache.shape[1], kcache.shape[3]
         Dv = vcache.shape[3]
         Hq = q.shape[1] // D
-        out = torch.empty(q.shape[0], Hq * Dv, dtype=q.dtype,
-                          device=q.device)
+        # padded rows of a ragged batch are never written by the kernel
+        out = (torch.zeros if lens is not None else torch.empty)(
+            q.shape[0], Hq * Dv, dtype=q.dtype, device=q.device)
+        splits, partials = 1, None
+        if T == 1:
+            splits = _attn_mod_splits(q.shape[0] * Hkv * -(-(Hq // Hkv) // 16),
+                                      kcache.shape[2])
+            if splits > 1:
+                partials = torch.empty(q.shape[0] * Hq * splits * (Dv + 2),
+                                       dtype=torch.float32, device=q.device)
         _native().attn_mod(q, kcache, vcache, pos, lens, slots, out, T,
                            scale, temp, softcap or 0.0, dist_r1, dist_r2,
-                           sinks, window or 0)
+                           sinks, window or 0, partials, splits)
         return out
     return ref.attn_mod(q, kcache, vcache, pos, T, scale, lens, slots, temp,
                         softcap, dist_r1, dist_r2, sinks, window)

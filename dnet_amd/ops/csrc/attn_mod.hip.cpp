@@ -96,17 +96,54 @@ struct ModParams {
   float scale, softcap;
 };
 
-template <typename T>
+// transcendental flavours: fp32 models use the accurate library functions,
+// bf16 models the hardware approximations (error far below bf16 rounding)
+template <bool FAST> __device__ __forceinline__ float m_exp(float x) {
+  return FAST ? __expf(x) : expf(x);
+}
+template <bool FAST> __device__ __forceinline__ float m_tanh(float x) {
+  return FAST ? 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f)
+              : tanhf(x);
+}
+template <bool FAST> __device__ __forceinline__ float m_log1p(float x) {
+  return FAST ? __logf(1.f + x) : log1pf(x);
+}
+
+// 16 B global -> LDS row copies (rows are 8 B aligned for bf16, 4 B for fp32)
+__device__ __forceinline__ void stage16(short* dst, const short* src, bool on) {
+  short8 z;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) z.x[j] = 0;
+  if (on) z = *reinterpret_cast<const short8*>(src);
+  *reinterpret_cast<short4v*>(dst) = *reinterpret_cast<short4v*>(&z.x[0]);
+  *reinterpret_cast<short4v*>(dst + 4) = *reinterpret_cast<short4v*>(&z.x[4]);
+}
+__device__ __forceinline__ void stage16(float* dst, const float* src, bool on) {
+  float4 z = {0.f, 0.f, 0.f, 0.f};
+  if (on) z = *reinterpret_cast<const float4*>(src);
+  dst[0] = z.x; dst[1] = z.y; dst[2] = z.z; dst[3] = z.w;
+}
+
+// VEC: head sizes are multiples of 16 B -> vector staging; for bf16 the
+// accumulate phase then owns output dims in pairs (one 4 B LDS read per key).
+// splits > 1 (decode only): blockIdx.x is the split; chunks are dealt round
+// robin and unnormalized (acc, m, l) go to `partial` [B, Hq, splits, DV+2].
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void attn_mod_rows(
     const T* __restrict__ q, const T* __restrict__ kc,
-    const T* __restrict__ vc, T* __restrict__ out, const ModParams P) {
+    const T* __restrict__ vc, T* __restrict__ out,
+    float* __restrict__ partial, const int splits, const ModParams P) {
+  constexpr bool FAST = sizeof(T) == 2;
+  constexpr bool PAIR = VEC && sizeof(T) == 2;
+  constexpr int EV = 16 / sizeof(T);
   const int b = blockIdx.z;
   const int G = P.Hq / P.Hkv;
   const int GS = (G + kRowsMax - 1) / kRowsMax;     // head-group splits
   const int hkv = blockIdx.y / GS;
   const int g0 = (blockIdx.y % GS) * kRowsMax;
   const int Gb = min(kRowsMax, G - g0);
-  const int t0 = blockIdx.x * P.QT;
+  const int split = splits > 1 ? blockIdx.x : 0;
+  const int t0 = splits > 1 ? 0 : blockIdx.x * P.QT;
   const int n = P.lens ? min(P.lens[b], P.T) : P.T;
   if (t0 >= n) return;
   const int slot = P.slots ? P.slots[b] : b;
@@ -149,6 +186,7 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[rr][j] = 0.f;
   }
+  const float cap = P.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
 
   const int kv_end = min(p0 + t0 + nt, P.Smax);          // exclusive
   const int kv_begin =
@@ -156,18 +194,33 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
   const int64_t kbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * D;
   const int64_t vbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * DV;
 
-  for (int s0 = kv_begin & ~(kChunkR - 1); s0 < kv_end; s0 += kChunkR) {
+  for (int s0 = (kv_begin & ~(kChunkR - 1)) + split * kChunkR; s0 < kv_end;
+       s0 += kChunkR * splits) {
     const int valid = min(kChunkR, kv_end - s0);
     __syncthreads();          // previous chunk consumed (and q staged)
-    for (int idx = threadIdx.x; idx < kChunkR * D; idx += blockDim.x) {
-      const int r = idx / D, e = idx % D;
-      k_lds[r * PK + e] =
-          r < valid ? kc[kbase + (int64_t)(s0 + r) * D + e] : (T)0;
-    }
-    for (int idx = threadIdx.x; idx < kChunkR * DV; idx += blockDim.x) {
-      const int r = idx / DV, e = idx % DV;
-      v_lds[r * PV + e] =
-          r < valid ? vc[vbase + (int64_t)(s0 + r) * DV + e] : (T)0;
+    if (VEC) {
+      const int dk = D / EV, dvv = DV / EV;
+      for (int idx = threadIdx.x; idx < kChunkR * dk; idx += blockDim.x) {
+        const int r = idx / dk, e = (idx % dk) * EV;
+        stage16(&k_lds[r * PK + e], &kc[kbase + (int64_t)(s0 + r) * D + e],
+                r < valid);
+      }
+      for (int idx = threadIdx.x; idx < kChunkR * dvv; idx += blockDim.x) {
+        const int r = idx / dvv, e = (idx % dvv) * EV;
+        stage16(&v_lds[r * PV + e], &vc[vbase + (int64_t)(s0 + r) * DV + e],
+                r < valid);
+      }
+    } else {
+      for (int idx = threadIdx.x; idx < kChunkR * D; idx += blockDim.x) {
+        const int r = idx / D, e = idx % D;
+        k_lds[r * PK + e] =
+            r < valid ? kc[kbase + (int64_t)(s0 + r) * D + e] : (T)0;
+      }
+      for (int idx = threadIdx.x; idx < kChunkR * DV; idx += blockDim.x) {
+        const int r = idx / DV, e = idx % DV;
+        v_lds[r * PV + e] =
+            r < valid ? vc[vbase + (int64_t)(s0 + r) * DV + e] : (T)0;
+      }
     }
     __syncthreads();
 #pragma unroll
@@ -179,26 +232,52 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
       bool live = lane < valid && j <= i;
       if (P.window > 0) live = live && (j > i - P.window);
       float s = dot_lds(&k_lds[lane * PK], &q_lds[r * PK], D) * tmp[rr];
-      if (P.softcap > 0.f) s = P.softcap * tanhf(s / P.softcap);
-      if (P.r1) s -= r1[rr] * log1pf(r2[rr] * (float)max(i - j, 0));
+      if (cap > 0.f) s = cap * m_tanh<FAST>(s * inv_cap);
+      if (P.r1) s -= r1[rr] * m_log1p<FAST>(r2[rr] * (float)max(i - j, 0));
       if (!live) s = -INFINITY;
       const float mn = fmaxf(m[rr], wave_all_max(s));
-      const float alpha = expf(m[rr] - mn);
-      const float p = live ? expf(s - mn) : 0.f;
+      const float alpha = m_exp<FAST>(m[rr] - mn);
+      const float p = live ? m_exp<FAST>(s - mn) : 0.f;
       l[rr] = l[rr] * alpha + wave_all_sum(p);
       m[rr] = mn;
       p_lds[wid * kChunkR + lane] = p;
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // wave-local slab
       const int vis = min(valid, i - s0 + 1);
+      const float* pw = &p_lds[wid * kChunkR];
+      if (PAIR) {
+        // lane owns dims (2*lane, 2*lane+1) + 128*jj
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int dv = lane + 64 * jj;
-        if (dv < DV) {
-          float a = acc[rr][jj] * alpha;
-          for (int s2 = 0; s2 < vis; ++s2)
-            a = fmaf(p_lds[wid * kChunkR + s2], ldv<T>(&v_lds[s2 * PV + dv]),
-                     a);
-          acc[rr][jj] = a;
+        for (int jj = 0; jj < 2; ++jj) {
+          const int dv = 2 * lane + 128 * jj;
+          if (dv < DV) {
+            float a0 = acc[rr][2 * jj] * alpha, a1 = acc[rr][2 * jj + 1] * alpha;
+            const short* vcol = reinterpret_cast<const short*>(v_lds) + dv;
+#pragma unroll 4
+            for (int s2 = 0; s2 < vis; ++s2) {
+              const unsigned pr =
+                  *reinterpret_cast<const unsigned*>(vcol + s2 * PV);
+              const float ps = pw[s2];
+              union { unsigned u; float f; } lo, hi;
+              lo.u = pr << 16;
+              hi.u = pr & 0xffff0000u;
+              a0 = fmaf(ps, lo.f, a0);
+              a1 = fmaf(ps, hi.f, a1);
+            }
+            acc[rr][2 * jj] = a0;
+            acc[rr][2 * jj + 1] = a1;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int dv = lane + 64 * jj;
+          if (dv < DV) {
+            float a = acc[rr][jj] * alpha;
+#pragma unroll 4
+            for (int s2 = 0; s2 < vis; ++s2)
+              a = fmaf(pw[s2], ldv<T>(&v_lds[s2 * PV + dv]), a);
+            acc[rr][jj] = a;
+          }
         }
       }
     }
@@ -209,20 +288,68 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
     const int r = wid + 4 * rr;
     if (r >= rows) continue;
     const int t = t0 + r / Gb, h = hkv * G + g0 + r % Gb;
+    if (splits > 1) {
+      float* pp = partial +
+                  (((int64_t)b * P.Hq + h) * splits + split) * (DV + 2);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        if (PAIR) {
+          const int dv = 2 * lane + 128 * (jj >> 1) + (jj & 1);
+          if (dv < DV) pp[dv] = acc[rr][jj];
+        } else {
+          const int dv = lane + 64 * jj;
+          if (dv < DV) pp[dv] = acc[rr][jj];
+        }
+      }
+      if (lane == 0) {
+        pp[DV] = m[rr];
+        pp[DV + 1] = l[rr];
+      }
+      continue;
+    }
     float c = 1.f;
     if (P.sinks) {
       const float sk = P.sinks[h];
       const float m2 = fmaxf(m[rr], sk);
-      c = expf(m[rr] - m2);
-      l[rr] = l[rr] * c + expf(sk - m2);
+      c = m_exp<FAST>(m[rr] - m2);
+      l[rr] = l[rr] * c + m_exp<FAST>(sk - m2);
     }
     const float inv = l[rr] > 0.f ? c / l[rr] : 0.f;
     T* op = out + ((int64_t)b * P.T + t) * P.Hq * DV + (int64_t)h * DV;
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
-      const int dv = lane + 64 * jj;
-      if (dv < DV) stv<T>(op + dv, acc[rr][jj] * inv);
+      if (PAIR) {
+        const int dv = 2 * lane + 128 * (jj >> 1) + (jj & 1);
+        if (dv < DV) stv<T>(op + dv, acc[rr][jj] * inv);
+      } else {
+        const int dv = lane + 64 * jj;
+        if (dv < DV) stv<T>(op + dv, acc[rr][jj] * inv);
+      }
     }
+  }
+}
+
+// merge the splits of one (batch row, head): one wave per output row
+template <typename T>
+__global__ __launch_bounds__(64) void attn_mod_combine(
+    const float* __restrict__ partial, T* __restrict__ out,
+    const float* __restrict__ sinks, const int* __restrict__ pos,
+    const int* __restrict__ slots, const int Hq, const int DV,
+    const int splits, const int Bc) {
+  const int b = blockIdx.x / Hq, h = blockIdx.x % Hq;
+  const float* pp = partial + (int64_t)blockIdx.x * splits * (DV + 2);
+  float M = -1e30f;
+  for (int s = 0; s < splits; ++s) M = fmaxf(M, pp[s * (DV + 2) + DV]);
+  if (sinks) M = fmaxf(M, sinks[h]);
+  float L = sinks ? expf(sinks[h] - M) : 0.f;
+  for (int s = 0; s < splits; ++s)
+    L += pp[s * (DV + 2) + DV + 1] * expf(pp[s * (DV + 2) + DV] - M);
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  for (int dv = threadIdx.x; dv < DV; dv += 64) {
+    float a = 0.f;
+    for (int s = 0; s < splits; ++s)
+      a += pp[s * (DV + 2) + dv] * expf(pp[s * (DV + 2) + DV] - M);
+    stv<T>(out + (int64_t)blockIdx.x * DV + dv, a * inv);
   }
 }
 
@@ -425,7 +552,8 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
               int64_t T, double scale, c10::optional<torch::Tensor> temp,
               double softcap, c10::optional<torch::Tensor> dist_r1,
               c10::optional<torch::Tensor> dist_r2,
-              c10::optional<torch::Tensor> sinks, int64_t window) {
+              c10::optional<torch::Tensor> sinks, int64_t window,
+              c10::optional<torch::Tensor> partials, int64_t splits) {
   DNET_CHECK(kcache.dim() == 4 && vcache.dim() == 4 &&
                  kcache.is_contiguous() && vcache.is_contiguous(), "cache");
   const int Bc = kcache.size(0), Hkv = kcache.size(1), Smax = kcache.size(2);
@@ -495,25 +623,42 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
 #undef AM
     return;
   }
-  if (f32) {
-    if (lds > 64 * 1024)
-      DNET_CHECK_HIP(hipFuncSetAttribute(
-          (const void*)attn_mod_rows<float>,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((attn_mod_rows<float>), grid, dim3(256), lds, stream,
-                       q.data_ptr<float>(), kcache.data_ptr<float>(),
-                       vcache.data_ptr<float>(), out.data_ptr<float>(), P);
-  } else {
-    if (lds > 64 * 1024)
-      DNET_CHECK_HIP(hipFuncSetAttribute(
-          (const void*)attn_mod_rows<short>,
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL((attn_mod_rows<short>), grid, dim3(256), lds, stream,
-                       (const short*)q.data_ptr(),
-                       (const short*)kcache.data_ptr(),
-                       (const short*)vcache.data_ptr(),
-                       (short*)out.data_ptr(), P);
+  // split-KV (decode only): more workgroups when batch x kv heads is small
+  int ns = (int)std::max<int64_t>(1, splits);
+  float* part = nullptr;
+  if (T != 1) ns = 1;
+  if (ns > 1) {
+    DNET_CHECK(partials.has_value() &&
+                   partials->scalar_type() == torch::kFloat32 &&
+                   partials->is_contiguous() &&
+                   partials->numel() >= B * Hq * ns * (int64_t)(DV + 2),
+               "partials fp32 [B, Hq, splits, DV+2]");
+    part = partials->data_ptr<float>();
   }
+  const dim3 rgrid(ns > 1 ? (unsigned)ns : grid.x, grid.y, grid.z);
+  const bool vec = (D * es) % 16 == 0 && (DV * es) % 16 == 0;
+#define AR(TT, VV)                                                          \
+  do {                                                                      \
+    if (lds > 64 * 1024)                                                    \
+      DNET_CHECK_HIP(hipFuncSetAttribute(                                   \
+          (const void*)attn_mod_rows<TT, VV>,                               \
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));           \
+    hipLaunchKernelGGL((attn_mod_rows<TT, VV>), rgrid, dim3(256), lds,      \
+                       stream, (const TT*)q.data_ptr(),                     \
+                       (const TT*)kcache.data_ptr(),                        \
+                       (const TT*)vcache.data_ptr(), (TT*)out.data_ptr(),   \
+                       part, ns, P);                                        \
+    if (ns > 1)                                                             \
+      hipLaunchKernelGGL((attn_mod_combine<TT>), dim3((unsigned)(B * Hq)),  \
+                         dim3(64), 0, stream, part, (TT*)out.data_ptr(),    \
+                         P.sinks, P.pos, P.slots, Hq, DV, ns, Bc);          \
+  } while (0)
+  if (f32) {
+    if (vec) AR(float, true); else AR(float, false);
+  } else {
+    if (vec) AR(short, true); else AR(short, false);
+  }
+#undef AR
 }
 
 }  // namespace dnet

@@ -85,7 +85,8 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
               int64_t T, double scale, c10::optional<torch::Tensor> temp,
               double softcap, c10::optional<torch::Tensor> dist_r1,
               c10::optional<torch::Tensor> dist_r2,
-              c10::optional<torch::Tensor> sinks, int64_t window);
+              c10::optional<torch::Tensor> sinks, int64_t window,
+              c10::optional<torch::Tensor> partials, int64_t splits);
 }  // namespace dnet
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {

@@ -81,6 +81,9 @@ CASES = [  # hq, hkv, d, dv, T, lens, pos0, slots, n_slots, smax
     (3, 3, 20, 12, 70, [70, 33], [64, 127], [1, 0], 2, 256),     # continued
     (32, 1, 32, 16, 9, [9, 4], [0, 3], None, 2, 80),             # G > 16
     (2, 2, 256, 256, 3, None, [10], None, 1, 70),
+    # decode against a long cache: the split-KV path and its combine
+    (8, 2, 64, 64, 1, None, [5, 300, 511, 0], None, 4, 600),
+    (6, 3, 40, 24, 1, None, [2000, 64, 1023], [2, 0, 1], 3, 2100),
     # prompts long enough for the matrix-core kernel (bf16), every tile class
     (8, 4, 64, 48, 200, [200, 77, 130], [0, 0, 0], [1, 2, 0], 3, 256),
     (4, 2, 192, 128, 70, [70, 3], [64, 10], None, 2, 160),
