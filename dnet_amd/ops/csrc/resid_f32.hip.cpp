@@ -22,7 +22,39 @@ template <typename T> __device__ __forceinline__ void stf(T* p, float v);
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void stf<short>(short* p, float v) { *p = f2bits(v); }
 
-template <typename TI, typename TO>
+// W-wide element groups: W = 4 when every row length is a multiple of 4
+// (16 B fp32 / 8 B bf16 accesses), else 1.
+template <int W> struct vecf { float v[W]; };
+template <int W, typename T>
+__device__ __forceinline__ vecf<W> ldw(const T* p) {
+  vecf<W> r;
+  if constexpr (W == 1) {
+    r.v[0] = ldf<T>(p);
+  } else if constexpr (sizeof(T) == 4) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+  } else {
+    const short4v t = *reinterpret_cast<const short4v*>(p);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r.v[j] = bits2f(t.x[j]);
+  }
+  return r;
+}
+template <int W, typename T>
+__device__ __forceinline__ void stw(T* p, const vecf<W>& r) {
+  if constexpr (W == 1) {
+    stf<T>(p, r.v[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4*>(p) = make_float4(r.v[0], r.v[1], r.v[2], r.v[3]);
+  } else {
+    short4v t;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t.x[j] = f2bits(r.v[j]);
+    *reinterpret_cast<short4v*>(p) = t;
+  }
+}
+
+template <typename TI, typename TO, int W>
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(
     const TI* __restrict__ x, const float* __restrict__ w, TO* __restrict__ y,
     const int N, const float eps) {
@@ -30,18 +62,24 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(
   const int64_t row = blockIdx.x;
   const TI* xr = x + row * N;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < N; i += blockDim.x) {
-    const float v = ldf<TI>(xr + i);
-    ss += v * v;
+  for (int i = threadIdx.x * W; i < N; i += blockDim.x * W) {
+    const vecf<W> v = ldw<W, TI>(xr + i);
+#pragma unroll
+    for (int j = 0; j < W; ++j) ss += v.v[j] * v.v[j];
   }
   ss = block_reduce_sum(ss, red);
   const float r = 1.0f / sqrtf(ss / (float)N + eps);
   TO* yr = y + row * N;
-  for (int i = threadIdx.x; i < N; i += blockDim.x)
-    stf<TO>(yr + i, ldf<TI>(xr + i) * r * w[i]);
+  for (int i = threadIdx.x * W; i < N; i += blockDim.x * W) {
+    vecf<W> v = ldw<W, TI>(xr + i);
+    const vecf<W> g = ldw<W, float>(w + i);
+#pragma unroll
+    for (int j = 0; j < W; ++j) v.v[j] = v.v[j] * r * g.v[j];
+    stw<W, TO>(yr + i, v);
+  }
 }
 
-template <typename T>
+template <typename T, int W>
 __global__ __launch_bounds__(256) void ls_resid_rmsnorm_kernel(
     float* __restrict__ h, const T* __restrict__ a, const float* __restrict__ s1,
     const T* __restrict__ b, const float* __restrict__ s2,
@@ -53,45 +91,65 @@ __global__ __launch_bounds__(256) void ls_resid_rmsnorm_kernel(
   const T* ar = a + row * N;
   const T* br = b ? b + row * N : nullptr;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < N; i += blockDim.x) {
-    float d = s1[i] * ldf<T>(ar + i);
-    if (br) d += s2[i] * ldf<T>(br + i);
-    const float v = hr[i] + d;
-    hr[i] = v;
-    ss += v * v;
+  for (int i = threadIdx.x * W; i < N; i += blockDim.x * W) {
+    vecf<W> hv = ldw<W, float>(hr + i);
+    const vecf<W> av = ldw<W, T>(ar + i), g1 = ldw<W, float>(s1 + i);
+    vecf<W> d;
+#pragma unroll
+    for (int j = 0; j < W; ++j) d.v[j] = g1.v[j] * av.v[j];
+    if (br) {
+      const vecf<W> bv = ldw<W, T>(br + i), g2 = ldw<W, float>(s2 + i);
+#pragma unroll
+      for (int j = 0; j < W; ++j) d.v[j] += g2.v[j] * bv.v[j];
+    }
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      hv.v[j] += d.v[j];
+      ss += hv.v[j] * hv.v[j];
+    }
+    stw<W, float>(hr + i, hv);
   }
   if (!wn) return;                       // uniform: residual update only
   ss = block_reduce_sum(ss, red);
   const float r = 1.0f / sqrtf(ss / (float)N + eps);
   T* yr = y + row * N;
   // each thread re-reads exactly the elements it wrote above
-  for (int i = threadIdx.x; i < N; i += blockDim.x)
-    stf<T>(yr + i, hr[i] * r * wn[i]);
+  for (int i = threadIdx.x * W; i < N; i += blockDim.x * W) {
+    vecf<W> hv = ldw<W, float>(hr + i);
+    const vecf<W> g = ldw<W, float>(wn + i);
+#pragma unroll
+    for (int j = 0; j < W; ++j) hv.v[j] = hv.v[j] * r * g.v[j];
+    stw<W, T>(yr + i, hv);
+  }
 }
 
 __device__ __forceinline__ float softplus_f(float t) {
   return t > 20.f ? t : log1pf(expf(t));
 }
 
-template <typename T>
+template <typename T, int W>
 __global__ __launch_bounds__(256) void xielu_kernel(
     const T* __restrict__ z, const float* __restrict__ pq, T* __restrict__ y,
     const int64_t n) {
   const float ap = softplus_f(pq[0]);
   const float an = 0.5f + softplus_f(pq[1]);
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    const float v = ldf<T>(z + i);
-    const float r = v > 0.f ? ap * v * v + 0.5f * v
-                            : an * (expm1f(v) - v) + 0.5f * v;
-    stf<T>(y + i, r);
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * W; i < n;
+       i += (int64_t)gridDim.x * blockDim.x * W) {
+    vecf<W> v = ldw<W, T>(z + i);
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      const float t = v.v[j];
+      v.v[j] = t > 0.f ? ap * t * t + 0.5f * t
+                       : an * (expm1f(t) - t) + 0.5f * t;
+    }
+    stw<W, T>(y + i, v);
   }
 }
 
 // qkv row layout: [q: nq*d | k: nkv*d | v: nkv*dv]. Token (b,t) = row b*T+t
 // sits at position pos[b]+t of cache row slots[b] (default b); tokens with
 // t >= lens[b] are padding: q is still written, the cache is not touched.
-template <typename T>
+template <typename T, int W>
 __global__ __launch_bounds__(256) void qknorm_append_kernel(
     const T* __restrict__ qkv, const float* __restrict__ qw,
     const float* __restrict__ kw, T* __restrict__ qout, T* __restrict__ kc,
@@ -115,25 +173,35 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
   const int64_t vbase = ((int64_t)slot * Hkv * Smax + p) * dv;
   if (!per_head) {
     float sq = 0.f, sk = 0.f;
-    for (int i = threadIdx.x; i < NQ; i += blockDim.x) {
-      const float v = ldf<T>(src + i);
-      sq += v * v;
+    for (int i = threadIdx.x * W; i < NQ; i += blockDim.x * W) {
+      const vecf<W> v = ldw<W, T>(src + i);
+#pragma unroll
+      for (int j = 0; j < W; ++j) sq += v.v[j] * v.v[j];
     }
-    for (int i = threadIdx.x; i < NK; i += blockDim.x) {
-      const float v = ldf<T>(src + NQ + i);
-      sk += v * v;
+    for (int i = threadIdx.x * W; i < NK; i += blockDim.x * W) {
+      const vecf<W> v = ldw<W, T>(src + NQ + i);
+#pragma unroll
+      for (int j = 0; j < W; ++j) sk += v.v[j] * v.v[j];
     }
     sq = block_reduce_sum(sq, red);
     sk = block_reduce_sum(sk, red);
     const float rq = 1.0f / sqrtf(sq / (float)NQ + eps);
     const float rk = 1.0f / sqrtf(sk / (float)NK + eps);
-    for (int i = threadIdx.x; i < NQ; i += blockDim.x)
-      stf<T>(qo + i, ldf<T>(src + i) * rq * qw[i]);
+    for (int i = threadIdx.x * W; i < NQ; i += blockDim.x * W) {
+      vecf<W> v = ldw<W, T>(src + i);
+      const vecf<W> g = ldw<W, float>(qw + i);
+#pragma unroll
+      for (int j = 0; j < W; ++j) v.v[j] = v.v[j] * rq * g.v[j];
+      stw<W, T>(qo + i, v);
+    }
     if (keep)
-      for (int i = threadIdx.x; i < NK; i += blockDim.x) {
-        const int hk = i / d, e = i % d;
-        stf<T>(kc + kbase + (int64_t)hk * Smax * d + e,
-               ldf<T>(src + NQ + i) * rk * kw[i]);
+      for (int i = threadIdx.x * W; i < NK; i += blockDim.x * W) {
+        const int hk = i / d, e = i % d;       // d % W == 0: no straddling
+        vecf<W> v = ldw<W, T>(src + NQ + i);
+        const vecf<W> g = ldw<W, float>(kw + i);
+#pragma unroll
+        for (int j = 0; j < W; ++j) v.v[j] = v.v[j] * rk * g.v[j];
+        stw<W, T>(kc + kbase + (int64_t)hk * Smax * d + e, v);
       }
   } else {
     // one wave per head; weights are per head-dim element
@@ -161,9 +229,10 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
     }
   }
   if (keep)
-    for (int i = threadIdx.x; i < NV; i += blockDim.x) {
+    for (int i = threadIdx.x * W; i < NV; i += blockDim.x * W) {
       const int hk = i / dv, e = i % dv;
-      vc[vbase + (int64_t)hk * Smax * dv + e] = src[NQ + NK + i];
+      stw<W, T>(vc + vbase + (int64_t)hk * Smax * dv + e,
+                ldw<W, T>(src + NQ + NK + i));
     }
 }
 
@@ -195,10 +264,17 @@ void rmsnorm_rows(torch::Tensor x, torch::Tensor w, torch::Tensor y,
   if (M == 0) return;
   auto st = current_stream();
   const float* wp = w.data_ptr<float>();
-#define RN(TI, TO)                                                         \
-  hipLaunchKernelGGL((rmsnorm_rows_kernel<TI, TO>), dim3(M), dim3(256), 0, \
-                     st, (const TI*)x.data_ptr(), wp, (TO*)y.data_ptr(), N, \
-                     (float)eps)
+#define RN(TI, TO)                                                          \
+  do {                                                                      \
+    if (N % 4 == 0)                                                         \
+      hipLaunchKernelGGL((rmsnorm_rows_kernel<TI, TO, 4>), dim3(M),         \
+                         dim3(256), 0, st, (const TI*)x.data_ptr(), wp,     \
+                         (TO*)y.data_ptr(), N, (float)eps);                 \
+    else                                                                    \
+      hipLaunchKernelGGL((rmsnorm_rows_kernel<TI, TO, 1>), dim3(M),         \
+                         dim3(256), 0, st, (const TI*)x.data_ptr(), wp,     \
+                         (TO*)y.data_ptr(), N, (float)eps);                 \
+  } while (0)
   if (is_f32(x) && is_f32(y)) RN(float, float);
   else if (is_f32(x) && is_bf16(y)) RN(float, short);
   else if (is_bf16(x) && is_bf16(y)) RN(short, short);
@@ -229,16 +305,17 @@ void ls_resid_rmsnorm(torch::Tensor h, torch::Tensor a, torch::Tensor s1,
                    y->scalar_type() == a.scalar_type(), "y shape/dtype");
   if (M == 0) return;
   auto st = current_stream();
-#define LR(TT)                                                              \
-  hipLaunchKernelGGL((ls_resid_rmsnorm_kernel<TT>), dim3(M), dim3(256), 0,  \
-                     st, h.data_ptr<float>(), (const TT*)a.data_ptr(),      \
+#define LR(TT, WW)                                                          \
+  hipLaunchKernelGGL((ls_resid_rmsnorm_kernel<TT, WW>), dim3(M), dim3(256), \
+                     0, st, h.data_ptr<float>(), (const TT*)a.data_ptr(),   \
                      s1.data_ptr<float>(),                                  \
                      b.has_value() ? (const TT*)b->data_ptr() : nullptr,    \
                      f32p(s2), f32p(wn),                                    \
                      y.has_value() ? (TT*)y->data_ptr() : nullptr, N,       \
                      (float)eps)
-  if (is_bf16(a)) LR(short);
-  else if (is_f32(a)) LR(float);
+  const bool v4 = N % 4 == 0;
+  if (is_bf16(a)) { if (v4) LR(short, 4); else LR(short, 1); }
+  else if (is_f32(a)) { if (v4) LR(float, 4); else LR(float, 1); }
   else DNET_CHECK(false, "ls_resid_rmsnorm: dtype");
 #undef LR
 }
@@ -250,17 +327,18 @@ void xielu(torch::Tensor z, torch::Tensor pq, torch::Tensor y) {
   DNET_CHECK(is_f32(pq) && pq.numel() == 2, "pq fp32 [2]");
   const int64_t n = z.numel();
   if (n == 0) return;
-  const int blocks = (int)std::min<int64_t>((n + 255) / 256, 256 * 16);
+  const bool v4 = n % 4 == 0;
+  const int64_t work = v4 ? n / 4 : n;
+  const int blocks = (int)std::min<int64_t>((work + 255) / 256, 256 * 16);
   auto st = current_stream();
-  if (is_bf16(z))
-    hipLaunchKernelGGL((xielu_kernel<short>), dim3(blocks), dim3(256), 0, st,
-                       (const short*)z.data_ptr(), pq.data_ptr<float>(),
-                       (short*)y.data_ptr(), n);
-  else if (is_f32(z))
-    hipLaunchKernelGGL((xielu_kernel<float>), dim3(blocks), dim3(256), 0, st,
-                       z.data_ptr<float>(), pq.data_ptr<float>(),
-                       y.data_ptr<float>(), n);
+#define XI(TT, WW)                                                          \
+  hipLaunchKernelGGL((xielu_kernel<TT, WW>), dim3(blocks), dim3(256), 0, st, \
+                     (const TT*)z.data_ptr(), pq.data_ptr<float>(),         \
+                     (TT*)y.data_ptr(), n)
+  if (is_bf16(z)) { if (v4) XI(short, 4); else XI(short, 1); }
+  else if (is_f32(z)) { if (v4) XI(float, 4); else XI(float, 1); }
   else DNET_CHECK(false, "xielu: dtype");
+#undef XI
 }
 
 void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
@@ -292,8 +370,9 @@ void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
   if (!slots.has_value()) DNET_CHECK(B <= Bc, "more rows than cache slots");
   if (M == 0) return;
   auto st = current_stream();
-#define QA(TT)                                                               \
-  hipLaunchKernelGGL((qknorm_append_kernel<TT>), dim3(M), dim3(256), 0, st,  \
+#define QA(TT, WW)                                                           \
+  hipLaunchKernelGGL((qknorm_append_kernel<TT, WW>), dim3(M), dim3(256), 0,  \
+                     st,                                                     \
                      (const TT*)qkv.data_ptr(), qw.data_ptr<float>(),        \
                      kw.data_ptr<float>(), (TT*)qout.data_ptr(),             \
                      (TT*)kcache.data_ptr(), (TT*)vcache.data_ptr(),         \
@@ -301,8 +380,9 @@ void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
                      (int)nq, (int)nkv, (int)d, (int)dv, (int)T, Bc, Hkv,     \
                      Smax,                                                   \
                      per_head)
-  if (is_bf16(qkv)) QA(short);
-  else if (is_f32(qkv)) QA(float);
+  const bool v4 = d % 4 == 0 && dv % 4 == 0;
+  if (is_bf16(qkv)) { if (v4) QA(short, 4); else QA(short, 1); }
+  else if (is_f32(qkv)) { if (v4) QA(float, 4); else QA(float, 1); }
   else DNET_CHECK(false, "qknorm_append: dtype");
 #undef QA
 }

@@ -514,3 +514,57 @@ def test_trace_replay_cli(tmp_path):
     close(rd(1), torch.stack([wa[9], wb[2]]))
     close(rd(2), wb[3:4])
     close(rd(3), wa[11:12])
+
+
+# ---------- pipeline stages (gloo, two processes) ----------
+
+def _ring_tokens():
+    g = torch.Generator().manual_seed(21)
+    return torch.randint(0, 97, (1, 2, 9), generator=g)
+
+
+def _ring_run(rank, world):
+    mc = ModelConfig.from_hf(make_cfg(BASE))
+    mc.compute_dtype = "float32"
+    ex = RingExecutor(mc, rank, world, "cpu", mb_count=1, mb_size=2, smax=64,
+                      seed=7, use_graphs=False)
+    first = ex.prefill(_ring_tokens())
+    gen = ex.decode_rounds(5)
+    return None if rank else torch.cat([first.unsqueeze(-1), gen], dim=-1)
+
+
+def _ring_rank_main(rank, world, port, q):
+    import os
+    os.environ.update(RANK=str(rank), WORLD_SIZE=str(world),
+                      MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port),
+                      LOCAL_RANK=str(rank))
+    import torch.distributed as dist
+    dist.init_process_group("gloo", rank=rank, world_size=world)
+    out = _ring_run(rank, world)
+    if rank == 0:
+        q.put(out)
+    dist.destroy_process_group()
+
+
+@pytest.mark.timeout(360)
+def test_two_stage_ring_matches_single():
+    """Layers split over two pipeline stages: the fp32 residual rides the
+    ring hops and the generated tokens equal the single-stage run."""
+    import multiprocessing as mp
+    import socket
+    single = _ring_run(0, 1)
+    s = socket.socket()
+    s.bind(("127.0.0.1", 0))
+    port = s.getsockname()[1]
+    s.close()
+    ctx = mp.get_context("spawn")
+    q = ctx.Queue()
+    procs = [ctx.Process(target=_ring_rank_main, args=(r, 2, port, q))
+             for r in range(2)]
+    for p in procs:
+        p.start()
+    out = q.get(timeout=150)
+    for p in procs:
+        p.join(timeout=60)
+        assert p.exitcode == 0
+    assert torch.equal(out, single)
