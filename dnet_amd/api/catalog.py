@@ -38,6 +38,10 @@ model_catalog: list[CatalogEntry] = [
                  tokenizer="byte"),
     CatalogEntry("deepseek-v3-lite-synthetic", preset="deepseek-v3-lite",
                  tokenizer="byte"),
+    CatalogEntry("posudra-tiny-random", preset="posudra-tiny",
+                 tokenizer="byte", ci_test=True),
+    CatalogEntry("posudra-8b-like-synthetic", preset="posudra-8b-like",
+                 tokenizer="byte"),
     CatalogEntry("openai/gpt-oss-20b", repo="openai/gpt-oss-20b"),
     CatalogEntry("deepseek-ai/DeepSeek-V2-Lite", repo="deepseek-ai/DeepSeek-V2-Lite"),
     # real checkpoints (local safetensors dir or pre-downloaded HF cache)

@@ -41,8 +41,16 @@ def main(argv=None) -> int:
     ap.add_argument("--no-graphs", action="store_true")
     args = ap.parse_args(argv)
 
+    if args.dtype == "float32":
+        # true fp32 products: no environment override may switch the vendor
+        # GEMM to a reduced-precision matrix mode
+        import os
+        os.environ.pop("TORCH_ALLOW_TF32_CUBLAS_OVERRIDE", None)
     import numpy as np
     import torch
+    if args.dtype == "float32":
+        torch.backends.cuda.matmul.allow_tf32 = False
+        torch.backends.cudnn.allow_tf32 = False
 
     on_gpu = torch.cuda.device_count() > 0      # else: CPU reference ops
     if on_gpu:
@@ -113,6 +121,13 @@ def main(argv=None) -> int:
                     rows.append(logits[slot_of[e["id"]]].view(1, -1))
                 length[e["id"]] += 1
             ex.slot_advance(rt._park_dev, rt._free_dev)
+            # a live request that sat this step out keeps its position (its
+            # row ran on a stale token; that append is overwritten by its
+            # real next token)
+            stepped = {slot_of[e["id"]] for e in entries}
+            for rid, s in slot_of.items():
+                if s not in stepped:
+                    ex.kvs[0].pos[s] = length[rid]
         elif entries:
             slots, prompts, want, start = [], [], [], []
             for e in entries:

@@ -474,16 +474,27 @@ def test_greedy_generation_through_slot_scheduler(tmp_path, device):
     rt._unload()
 
 
+@pytest.mark.gpu
+def test_trace_replay_cli_gpu(tmp_path):
+    """The same replay on the GPU box (HIP kernels, captured decode graph,
+    slot batch grown after capture)."""
+    test_trace_replay_cli(tmp_path)
+
+
 def test_trace_replay_cli(tmp_path):
     """bin/trace_run end to end on a tiny checkpoint: a prompt batch of
-    unequal requests, decode steps, a request that ends early."""
+    unequal requests (more of them than the initial slot count, so the slot
+    batch grows), decode steps, a request that sits a step out, requests
+    that end early."""
     cfg = make_cfg(BASE[:2], vocab=53)
     sd = make_weights(cfg, 16)
     write_checkpoint(tmp_path / "m", cfg, sd)
     a, b = tokens(12, 53, 1).tolist(), tokens(4, 53, 2).tolist()
+    c = tokens(7, 53, 3).tolist()
     steps = [
         {"step": 0, "entries": [{"id": "a", "tokens": a[:9], "want": [0, 8]},
-                                {"id": "b", "tokens": b[:2], "want": []}],
+                                {"id": "b", "tokens": b[:2], "want": []},
+                                {"id": "c", "tokens": c[:5], "want": [4]}],
          "end": []},
         {"step": 1, "entries": [{"id": "a", "tokens": a[9:10], "want": [0]},
                                 {"id": "b", "tokens": b[2:3], "want": [0]}],
@@ -493,27 +504,34 @@ def test_trace_replay_cli(tmp_path):
          "end": ["b"]},
         {"step": 3, "entries": [{"id": "a", "tokens": a[11:12], "want": [0]}],
          "end": ["a"]},
+        {"step": 4, "entries": [{"id": "c", "tokens": c[5:6], "want": [0]}],
+         "end": []},
+        {"step": 5, "entries": [{"id": "c", "tokens": c[6:7], "want": [0]}],
+         "end": ["c"]},
     ]
     root = Path(__file__).resolve().parents[1]
     r = subprocess.run(
         [sys.executable, str(root / "bin" / "trace_run"), "--model",
          str(tmp_path / "m"), "--dtype", "float32", "--out",
-         str(tmp_path / "out"), "--max-tokens", "32"],
+         str(tmp_path / "out"), "--max-tokens", "32", "--max-batch", "2"],
         input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
         capture_output=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [
-        f"done {i}" for i in range(4)]
+        f"done {i}" for i in range(6)]
     wa, wb = O.forward(a, cfg, sd), O.forward(b, cfg, sd)
+    wc = O.forward(c, cfg, sd)
     import numpy as np
 
     def rd(i):
         return torch.from_numpy(np.fromfile(tmp_path / "out" / f"{i}.f32",
                                             dtype="<f4").reshape(-1, 53))
-    close(rd(0), wa[[0, 8]])
+    close(rd(0), torch.cat([wa[[0, 8]], wc[4:5]]))
     close(rd(1), torch.stack([wa[9], wb[2]]))
     close(rd(2), wb[3:4])
     close(rd(3), wa[11:12])
+    close(rd(4), wc[5:6])
+    close(rd(5), wc[6:7])
 
 
 # ---------- pipeline stages (gloo, two processes) ----------
