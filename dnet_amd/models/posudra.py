@@ -217,9 +217,12 @@ class PosudraRingModel(RingModel):
             f = None
             if lw.up is not None:
                 f = lw.down(ops.xielu(lw.up(u), lw.act_pq))
-            nxt = (self._layer(layer_ids[i + 1]).attn_norm
-                   if i + 1 < len(layer_ids) else None)
-            # residual update fused with the next layer's norm
+            # residual update fused with the next layer's norm (resident
+            # layers only: binding the next layer of a streamed window here
+            # could recycle the slot this layer's scales still live in)
+            nxt = (self.layers[layer_ids[i + 1]].attn_norm
+                   if i + 1 < len(layer_ids)
+                   and layer_ids[i + 1] in self.layers else None)
             u = ops.ls_resid_rmsnorm(x, o, lw.ls1, f, lw.ls2, nxt, eps, wdt)
             if self._obs_sync:
                 self._profile_layer_sync(lid)

@@ -586,3 +586,18 @@ def test_two_stage_ring_matches_single():
         p.join(timeout=60)
         assert p.exitcode == 0
     assert torch.equal(out, single)
+
+
+def test_streamed_weights_match_resident():
+    """Windowed weight residency (layers streamed through two device slots)
+    generates the same tokens as the fully resident model."""
+    cfg = make_cfg([(mixer(4, 2, 16, 8), 40)] * 4)
+    toks = torch.randint(0, 97, (1, 2, 9),
+                         generator=torch.Generator().manual_seed(1))
+    outs = []
+    for residency in (0, 2):
+        ex = RingExecutor(ModelConfig.from_hf(cfg), 0, 1, "cpu", mb_size=2,
+                          smax=64, residency=residency, use_graphs=False)
+        first = ex.prefill(toks)
+        outs.append(torch.cat([first.unsqueeze(-1), ex.decode_rounds(4)], -1))
+    assert torch.equal(outs[0], outs[1])
