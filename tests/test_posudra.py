@@ -601,3 +601,28 @@ def test_streamed_weights_match_resident():
         first = ex.prefill(toks)
         outs.append(torch.cat([first.unsqueeze(-1), ex.decode_rounds(4)], -1))
     assert torch.equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_awkward_sizes(device, dtype):
+    """Widths and head sizes that are not multiples of the kernels' vector
+    widths or tile sizes: every scalar / padded code path against the
+    oracle, in a prompt batch and in decoding."""
+    for width, ff, layers in (
+            (100, 77, [(mixer(6, 3, 24, 40), 77), (mixer(2, 1, 10, 6), None)]),
+            (90, 36, [(mixer(5, 1, 7, 9, softcap=2.0), 36)] * 2),
+            (72, 200, [(mixer(3, 3, 72, 136), 200)])):
+        cfg = make_cfg(layers, width=width, vocab=131)
+        sd = make_weights(cfg, width)
+        ex = executor(cfg, sd, device, dtype, slots=3, smax=160)
+        a, b = tokens(80, 131, 1), tokens(23, 131, 2)
+        wa, wb = O.forward(a, cfg, sd), O.forward(b, cfg, sd)
+        got = ex.prefill_slots([2, 0], [a[:70], b[:20]],
+                               want=[[0, 31, 32, 63, 64, 69], [0, 19]])
+        close(got[0], wa[[0, 31, 32, 63, 64, 69]], dtype)
+        close(got[1], wb[[0, 19]], dtype)
+        for i in range(3):
+            lg = decode_steps(ex, {2: a[70 + i], 0: b[20 + i]})
+            close(lg[2:3], wa[70 + i].view(1, -1), dtype)
+            close(lg[0:1], wb[20 + i].view(1, -1), dtype)
