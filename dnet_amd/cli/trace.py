@@ -73,6 +73,9 @@ def main(argv=None) -> int:
         return 3
     smax = (max(args.max_tokens, 16) + 63) // 64 * 64 + 64
     rt = ShardRuntime("trace")
+    # a replay keeps nothing but compiled code between calls: no repacked
+    # per-layer weight cache is written or read
+    rt.settings.storage.repack_on_load = False
     if args.no_graphs:
         rt.settings.compute.use_graphs = False
     rt._load(ShardLoadModelRequest(

@@ -56,7 +56,8 @@ class PosudraRingModel(RingModel):
                 "posudra: tensor/context parallelism inside a stage is not "
                 "implemented (pipeline stages are)")
         assert cfg.layer_specs is not None, "posudra needs per-layer specs"
-        assert cfg.quant is None, "posudra: weight quantization not wired"
+        assert cfg.quant is None or cfg.quant.fmt != "mxfp4", \
+            "posudra: grouped int8/int4 weights only"
         super().__init__(cfg, layer_ids, device, is_first, is_last,
                          smax=smax, **kw)
         self.wdtype = (torch.float32 if cfg.compute_dtype == "float32"
@@ -84,6 +85,13 @@ class PosudraRingModel(RingModel):
     # ---------- weights ----------
 
     def _lin(self, w: torch.Tensor) -> Linear:
+        q = self.cfg.quant
+        if (q is not None and self.wdtype == torch.bfloat16
+                and w.shape[1] % max(q.group, 128) == 0):
+            # grouped int8/int4 weights through the framework's fused
+            # dequant GEMMs (projections whose K does not fit stay bf16)
+            return Linear.make(w.to(torch.bfloat16).to(self.device)
+                               .contiguous(), None, q)
         return Linear(w.to(self.wdtype).to(self.device).contiguous())
 
     def _vec(self, t: torch.Tensor) -> torch.Tensor:

@@ -431,7 +431,8 @@ def oracle_greedy(prompt, n, cfg, sd):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-def test_greedy_generation_through_slot_scheduler(tmp_path, device):
+def test_greedy_generation_through_slot_scheduler(tmp_path, device,
+                                                  monkeypatch):
     """Checkpoint on disk -> ShardRuntime load (metadata buckets, weight
     load, slots) -> three concurrent requests of unequal prompts admitted
     as one ragged batch -> greedy tokens equal the oracle's."""
@@ -451,6 +452,8 @@ def test_greedy_generation_through_slot_scheduler(tmp_path, device):
             pass
 
     rt = ShardRuntime("probe")
+    # (no repacked-weights cache keyed by a recycled temporary path)
+    monkeypatch.setattr(rt.settings.storage, "repack_on_load", False)
     rt._load(ShardLoadModelRequest(
         model_path=str(tmp_path / "m"), total_layers=4, layers=[0, 1, 2, 3],
         max_batch=3, max_seq=128, dtype="float32"))
@@ -626,3 +629,25 @@ def test_awkward_sizes(device, dtype):
             lg = decode_steps(ex, {2: a[70 + i], 0: b[20 + i]})
             close(lg[2:3], wa[70 + i].view(1, -1), dtype)
             close(lg[0:1], wb[20 + i].view(1, -1), dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_int8_weights(device):
+    """Grouped int8 weights (the framework's W8A16 linears) stay within
+    quantization error of the oracle on the unquantized weights."""
+    from dnet_amd.models import QuantConfig
+    cfg = make_cfg([(mixer(4, 2, 32, 32), 256)] * 2, width=128, vocab=101)
+    sd = make_weights(cfg, 31)
+    mc = ModelConfig.from_hf(cfg, quant=QuantConfig(8, 128))
+    ex = RingExecutor(mc, 0, 1, device, mb_size=2, smax=96,
+                      init_weights=False, use_graphs=False)
+    ex.model.load_state_dict(sd)
+    assert ex.model.layers[0].qkv.is_quant and ex.model.layers[0].down.is_quant
+    toks = tokens(40, 101, 5)
+    want = O.forward(toks, cfg, sd)
+    got = ex.prefill_slots([0], [toks[:36]], want=[[0, 35]])[0]
+    scale = float(want.float().pow(2).mean().sqrt())
+    assert float((got.float().cpu() - want[[0, 35]].float()).abs().max()) \
+        < 0.2 * scale
+    lg = decode_steps(ex, {0: toks[36]})
+    assert float((lg[0] - want[36].float()).abs().max()) < 0.2 * scale
