@@ -117,7 +117,12 @@ def main(argv=None) -> int:
             for e in entries:
                 toks[slot_of[e["id"]]] = int(e["tokens"][0])
             ex.tokbuf[0].copy_(toks)
-            ex.slot_step_compute()
+            # rows that sit this step out (free slots, live requests without
+            # an entry) run as idle rows: their recurrent state is kept
+            stepped = {slot_of[e["id"]] for e in entries}
+            idle = torch.ones(ex.mb_size, dtype=torch.bool)
+            idle[sorted(stepped)] = False
+            ex.slot_step_compute(park=idle.to(ex.device))
             logits = ex.logits_buf[0].float()
             for e in entries:
                 if e.get("want"):
@@ -127,7 +132,6 @@ def main(argv=None) -> int:
             # a live request that sat this step out keeps its position (its
             # row ran on a stale token; that append is overwritten by its
             # real next token)
-            stepped = {slot_of[e["id"]] for e in entries}
             for rid, s in slot_of.items():
                 if s not in stepped:
                     ex.kvs[0].pos[s] = length[rid]

@@ -43,5 +43,9 @@ from .posudra import PosudraRingModel  # noqa: E402
 
 register(PosudraRingModel)
 
-__all__ = ["ModelConfig", "QuantConfig", "RingModel", "MoERingModel", "KVCache", "PosudraRingModel",
+from .gegorax import GegoraxRingModel  # noqa: E402
+
+register(GegoraxRingModel)
+
+__all__ = ["GegoraxRingModel", "ModelConfig", "QuantConfig", "RingModel", "MoERingModel", "KVCache", "PosudraRingModel",
            "Linear", "PRESETS", "get_ring_model", "register"]

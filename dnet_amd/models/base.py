@@ -283,7 +283,8 @@ class KVCache:
     def __init__(self, cfg: ModelConfig, layer_ids: Sequence[int], batch: int,
                  smax: int, device, kv_bits: int = 16,
                  layer_dims: Optional[Sequence[tuple]] = None,
-                 dtype: torch.dtype = torch.bfloat16):
+                 dtype: torch.dtype = torch.bfloat16,
+                 layer_state: Optional[Sequence[dict]] = None):
         self.layer_ids = list(layer_ids)
         self.local = {g: i for i, g in enumerate(self.layer_ids)}
         self.kv_bits = kv_bits
@@ -292,15 +293,31 @@ class KVCache:
         self.smax = smax
         self.batch = batch
         self.kscale = self.vscale = None
+        # rows that sit a slot-batch decode step out (free or mid-prefill
+        # slots): sequence-state models leave their state untouched
+        self.idle = torch.zeros(batch, dtype=torch.bool, device=device)
+        # per-layer sequence state beside (or instead of) keys and values:
+        # one dict name -> tensor [B, ...] per local layer (recurrent
+        # states, convolution tails, pooled-block caches)
+        self.state: list = [{} for _ in range(L)]
+        if layer_state is not None:
+            assert len(layer_state) == L
+            self.state = [
+                {n: torch.zeros(batch, *shape, dtype=dt, device=device)
+                 for n, (shape, dt) in (ls or {}).items()}
+                for ls in layer_state]
         if layer_dims is not None:
             # heterogeneous stacks: one (kv_heads, k_dim, v_dim) per local
             # layer -> per-layer tensors [B, Hkv_l, Smax, D_l] (self.k[li]
-            # indexes a list instead of a stacked tensor's first axis)
+            # indexes a list instead of a stacked tensor's first axis); a
+            # layer without attention has None
             assert kv_bits == 16 and len(layer_dims) == L
-            self.k = [torch.zeros(batch, hk, smax, dk, dtype=dtype,
-                                  device=device) for hk, dk, _ in layer_dims]
-            self.v = [torch.zeros(batch, hk, smax, dv, dtype=dtype,
-                                  device=device) for hk, _, dv in layer_dims]
+            self.k = [None if t is None else
+                      torch.zeros(batch, t[0], smax, t[1], dtype=dtype,
+                                  device=device) for t in layer_dims]
+            self.v = [None if t is None else
+                      torch.zeros(batch, t[0], smax, t[2], dtype=dtype,
+                                  device=device) for t in layer_dims]
             return
         shape = (L, batch, cfg.num_kv_heads, smax, cfg.head_dim)
         if kv_bits == 8:
@@ -321,9 +338,12 @@ class KVCache:
         their state (continuous batching)."""
         import copy
         c = copy.copy(self)
+        c.idle = self.idle[s:s + 1]
+        c.state = [{n: t[s:s + 1] for n, t in st.items()}
+                   for st in self.state]
         if isinstance(self.k, list):
-            c.k = [t[s:s + 1] for t in self.k]
-            c.v = [t[s:s + 1] for t in self.v]
+            c.k = [None if t is None else t[s:s + 1] for t in self.k]
+            c.v = [None if t is None else t[s:s + 1] for t in self.v]
             c.pos = self.pos[s:s + 1]
             c.batch = 1
             return c
@@ -348,9 +368,12 @@ class KVCache:
             shape[axis] = extra
             return torch.cat([t, torch.zeros(shape, dtype=t.dtype,
                                              device=t.device)], dim=axis)
+        self.state = [{n: pad(t, 0) for n, t in st.items()}
+                      for st in self.state]
+        self.idle = pad(self.idle, 0)
         if isinstance(self.k, list):
-            self.k = [pad(t, 0) for t in self.k]
-            self.v = [pad(t, 0) for t in self.v]
+            self.k = [None if t is None else pad(t, 0) for t in self.k]
+            self.v = [None if t is None else pad(t, 0) for t in self.v]
         else:
             self.k, self.v = pad(self.k, 1), pad(self.v, 1)
             if self.kscale is not None:
@@ -379,8 +402,11 @@ class KVCache:
         self.pos.zero_()
 
     def nbytes(self) -> int:
+        extra = sum(t.numel() * t.element_size()
+                    for st in self.state for t in st.values())
         if isinstance(self.k, list):
-            return sum(t.numel() * t.element_size() for t in self.k + self.v)
+            return extra + sum(t.numel() * t.element_size()
+                               for t in self.k + self.v if t is not None)
         n = 2 * self.k.numel() * self.k.element_size()
         if self.kscale is not None:
             n += 2 * self.kscale.numel() * self.kscale.element_size()

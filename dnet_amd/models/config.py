@@ -69,6 +69,9 @@ class ModelConfig:
     # num_q_heads / head_dim / ... above then hold layer 0's sizes
     layer_specs: Optional[list] = None
     embedding_scale: float = 1.0
+    # per-layer token input (gegorax): width of each layer's slice of the
+    # second embedding table; 0 = none
+    token_side_dim: int = 0
     # "bfloat16": bf16 weights/activations with 32-bit accumulation;
     # "float32": weights, activations and matrix products in true fp32
     # (honoured by the model families that implement it)
@@ -114,10 +117,78 @@ class ModelConfig:
         )
 
     @classmethod
+    def from_gegorax(cls, cfg: dict,
+                     quant: Optional[QuantConfig] = None) -> "ModelConfig":
+        """Gegorax checkpoints list their layers: {"architecture":
+        "Gegorax", "vocab", "width", "norm": {"eps"}, "token_side":
+        {"dim"} (optional), "layers": [{"type": "parallel" |
+        "general_delta", "mixer": {...}, "mlp": {"kind": "dense" | "moe",
+        ...} | null}, ...]}. Every size and constant is per layer."""
+        specs = [dict(s) for s in cfg["layers"]]
+        att = None
+        for i, s in enumerate(specs):
+            kind, m = s.get("type"), s.get("mixer") or {}
+            if kind == "parallel":
+                need = {"left": ("heads", "kv_heads", "dim", "vdim", "scale"),
+                        "right": ("conv", "groups", "heads", "norm_groups",
+                                  "state", "vdim")}
+                for side, keys in need.items():
+                    missing = [k for k in keys if k not in (m.get(side) or {})]
+                    if missing:
+                        raise ValueError(f"gegorax layer {i}: mixer.{side} "
+                                         f"lacks {missing}")
+                lf, rt = m["left"], m["right"]
+                if lf["heads"] % lf["kv_heads"] or rt["heads"] % rt["groups"] \
+                        or (rt["heads"] * rt["vdim"]) % rt["norm_groups"]:
+                    raise ValueError(f"gegorax layer {i}: head counts do "
+                                     "not divide")
+                mask = lf.get("mask") or {}
+                if mask.get("pool") and not mask.get("size"):
+                    raise ValueError(f"gegorax layer {i}: pooled blocks "
+                                     "need a window size")
+                att = att or lf
+            elif kind == "general_delta":
+                if "heads" not in m or "dim" not in m:
+                    raise ValueError(f"gegorax layer {i}: mixer lacks "
+                                     "heads/dim")
+            else:
+                raise ValueError(f"gegorax layer {i}: unknown mixer type "
+                                 f"{kind!r}")
+            ff = s.get("mlp")
+            if ff is not None and ff.get("kind") not in ("dense", "moe"):
+                raise ValueError(f"gegorax layer {i}: unknown feed-forward "
+                                 f"kind {ff.get('kind')!r}")
+        att = att or {}
+        ffs = [s["mlp"]["ff"] for s in specs
+               if s.get("mlp") and s["mlp"].get("kind") == "dense"]
+        moe = [s["mlp"] for s in specs
+               if s.get("mlp") and s["mlp"].get("kind") == "moe"]
+        return cls(
+            model_type="gegorax",
+            hidden_size=cfg["width"],
+            num_layers=len(specs),
+            num_q_heads=att.get("heads", 1),
+            num_kv_heads=att.get("kv_heads", 1),
+            head_dim=att.get("dim", 1),
+            v_head_dim=att.get("vdim", 1),
+            intermediate_size=max(ffs) if ffs else 0,
+            num_experts=max((m["router"]["experts"] for m in moe), default=0),
+            num_experts_per_tok=max((m["router"]["top"] for m in moe),
+                                    default=0),
+            vocab_size=cfg["vocab"],
+            rms_eps=cfg["norm"]["eps"],
+            token_side_dim=int((cfg.get("token_side") or {}).get("dim", 0)),
+            layer_specs=specs,
+            quant=quant,
+        )
+
+    @classmethod
     def from_hf(cls, cfg: dict, quant: Optional[QuantConfig] = None) -> "ModelConfig":
-        if str(cfg.get("architecture", "")).lower() == "posudra" \
-                or cfg.get("model_type") == "posudra":
+        arch = str(cfg.get("architecture", "")).lower()
+        if arch == "posudra" or cfg.get("model_type") == "posudra":
             return cls.from_posudra(cfg, quant)
+        if arch == "gegorax" or cfg.get("model_type") == "gegorax":
+            return cls.from_gegorax(cfg, quant)
         mt = cfg.get("model_type", "llama")
         hidden = cfg["hidden_size"]
         nq = cfg.get("num_attention_heads", 32)
@@ -188,6 +259,44 @@ def posudra_config(width: int, layers: int, heads: int, kv_heads: int,
             "layers": [dict(layer) for _ in range(layers)]}
 
 
+def gegorax_config(width: int, layers: int, vocab: int, heads: int,
+                   kv_heads: int, dim: int, vdim: int, window: int, pool: int,
+                   ssm_heads: int, ssm_vdim: int, ssm_state: int,
+                   delta_heads: int, delta_dim: int, ff: int,
+                   experts: int = 0, top: int = 0, expert_ff: int = 0,
+                   shared_ff: int = 0, side_dim: int = 0,
+                   pattern: str = "pd", rot_base: float = 10000.0,
+                   eps: float = 1e-6) -> dict:
+    """A gegorax stack in the checkpoint's config.json layout. ``pattern``
+    repeats over the layers: 'p' = attention + state-space side by side,
+    'd' = generalized delta rule; every second layer's feed-forward is a
+    mixture of experts when ``experts`` > 0, dense otherwise."""
+    par = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim,
+                    "vdim": vdim, "scale": dim ** -0.5,
+                    "mask": {"size": window, "pool": pool},
+                    "rot": {"dims": dim, "base": rot_base}},
+           "right": {"conv": 4, "groups": max(1, ssm_heads // 8),
+                     "heads": ssm_heads, "norm_groups": 1,
+                     "state": ssm_state, "vdim": ssm_vdim}}
+    dl = {"heads": delta_heads, "dim": delta_dim}
+    dense = {"kind": "dense", "ff": ff} if ff else None
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top},
+           "expert": {"ff": expert_ff, "limit": 7.0}}
+    if shared_ff:
+        moe["shared"] = {"ff": shared_ff, "limit": 7.0}
+    out = []
+    for i in range(layers):
+        t = pattern[i % len(pattern)]
+        out.append({"type": "parallel" if t == "p" else "general_delta",
+                    "mixer": par if t == "p" else dl,
+                    "mlp": moe if (experts and i % 2 == 1) else dense})
+    cfg = {"architecture": "Gegorax", "vocab": vocab, "width": width,
+           "norm": {"eps": eps}, "layers": out}
+    if side_dim:
+        cfg["token_side"] = {"dim": side_dim}
+    return cfg
+
+
 # Known configs for synthetic benchmarking (random-init weights; no network).
 PRESETS: dict[str, dict] = {
     "llama-3-8b": dict(model_type="llama", hidden_size=4096, num_hidden_layers=32,
@@ -250,6 +359,9 @@ PRESETS: dict[str, dict] = {
                                       151936),
     "posudra-tiny": posudra_config(128, 4, 4, 2, 32, 16, 192, 256,
                                    softcap=8.0, embedding_scale=4.0),
+    "gegorax-tiny": gegorax_config(128, 4, 256, 4, 2, 32, 16, 24, 4, 4, 16,
+                                   16, 2, 32, 192, experts=6, top=2,
+                                   expert_ff=64, shared_ff=64, side_dim=16),
     "tiny": dict(model_type="llama", hidden_size=128, num_hidden_layers=4,
                  num_attention_heads=2, num_key_value_heads=2, head_dim=64,
                  intermediate_size=256, vocab_size=256, rope_theta=10000.0),

@@ -474,15 +474,19 @@ def qknorm_append(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor,
                   eps: float, nq: int, nkv: int, d: int, dv: int,
                   kcache: torch.Tensor, vcache: torch.Tensor,
                   pos: torch.Tensor, T: int, lens=None, slots=None,
-                  per_head: bool = False) -> torch.Tensor:
+                  per_head: bool = False,
+                  rot_freq: torch.Tensor | None = None) -> torch.Tensor:
+    """``rot_freq`` fp32 [n] (per-head norm only): interleaved channel pairs
+    (2i, 2i+1), i < n, turn by position * rot_freq[i] after the norm."""
     if qkv.is_cuda:
         q = torch.empty(qkv.shape[0], nq * d, dtype=qkv.dtype,
                         device=qkv.device)
         _native().qknorm_append(qkv, qw, kw, q, kcache, vcache, pos, lens,
-                                slots, eps, nq, nkv, d, dv, T, per_head)
+                                slots, eps, nq, nkv, d, dv, T, per_head,
+                                rot_freq)
         return q
     return ref.qknorm_append(qkv, qw, kw, eps, nq, nkv, d, dv, kcache,
-                             vcache, pos, T, lens, slots, per_head)
+                             vcache, pos, T, lens, slots, per_head, rot_freq)
 
 
 def _attn_mod_splits(blocks: int, smax: int) -> int:
@@ -498,11 +502,17 @@ def _attn_mod_splits(blocks: int, smax: int) -> int:
 def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
              pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
              temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
-             sinks=None, window: int = 0) -> torch.Tensor:
+             sinks=None, window: int = 0, pool_k=None, pool_v=None,
+             pool: int = 0) -> torch.Tensor:
     """Causal attention against the cache with per-head temperature, tanh
     soft cap, logarithmic distance penalty and a sink in the softmax
     denominator (each optional). One entry point for decode (T=1) and
-    ragged batched prefill (T = padded length, lens = real lengths)."""
+    ragged batched prefill (T = padded length, lens = real lengths).
+    ``window`` > 0 limits the tokens seen to the last ``window``; with
+    ``pool`` > 0 every whole block of ``pool`` positions before the window
+    is seen as one entry of the pooled caches (see ``kv_pool_update``)."""
+    if pool:
+        assert window and pool_k is not None and pool_v is not None
     if q.is_cuda:
         Hkv, D = kcache.shape[1], kcache.shape[3]
         Dv = vcache.shape[3]
@@ -512,14 +522,133 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
             q.shape[0], Hq * Dv, dtype=q.dtype, device=q.device)
         splits, partials = 1, None
         if T == 1:
+            # a windowed row scans at most window + pooled entries
+            span = kcache.shape[2]
+            if window:
+                span = min(span, window + 64
+                           + (pool_k.shape[2] if pool else 0))
             splits = _attn_mod_splits(q.shape[0] * Hkv * -(-(Hq // Hkv) // 16),
-                                      kcache.shape[2])
+                                      span)
             if splits > 1:
                 partials = torch.empty(q.shape[0] * Hq * splits * (Dv + 2),
                                        dtype=torch.float32, device=q.device)
         _native().attn_mod(q, kcache, vcache, pos, lens, slots, out, T,
                            scale, temp, softcap or 0.0, dist_r1, dist_r2,
-                           sinks, window or 0, partials, splits)
+                           sinks, window or 0, partials, splits,
+                           pool_k if pool else None,
+                           pool_v if pool else None, pool or 0)
         return out
     return ref.attn_mod(q, kcache, vcache, pos, T, scale, lens, slots, temp,
-                        softcap, dist_r1, dist_r2, sinks, window)
+                        softcap, dist_r1, dist_r2, sinks, window, pool_k,
+                        pool_v, pool)
+
+
+# ---- pooled-block caches, short convolutions, linear recurrences ----
+# Sequence-state mixers (gegorax): csrc/seq_state.hip.cpp and
+# csrc/row_fused.hip.cpp. Recurrent state, decays, step sizes and gates of
+# the recurrences are fp32 whatever the activation dtype.
+
+def kv_pool_update(kcache, vcache, pool_k, pool_v, pos, T: int, pool: int,
+                   lens=None, slots=None) -> None:
+    if kcache.is_cuda:
+        _native().kv_pool_update(kcache, vcache, pool_k, pool_v, pos, lens,
+                                 slots, T, pool)
+        return
+    ref.kv_pool_update(kcache, vcache, pool_k, pool_v, pos, T, pool, lens,
+                       slots)
+
+
+def causal_conv_silu(x, col0: int, w, bias, state, pos, T: int, lens=None,
+                     slots=None) -> torch.Tensor:
+    if x.is_cuda:
+        y = torch.empty(x.shape[0], w.shape[0], dtype=torch.float32,
+                        device=x.device)
+        _native().causal_conv_silu(x, col0, w, bias, state, y, pos, lens,
+                                   slots, T)
+        return y
+    return ref.causal_conv_silu(x, col0, w, bias, state, pos, T, lens, slots)
+
+
+def ssd_scan(xbc, dt_src, dt_col0: int, dt_bias, a_log, dskip, state, pos,
+             T: int, heads: int, P: int, N: int, G: int, lens=None,
+             slots=None) -> torch.Tensor:
+    if xbc.is_cuda:
+        # padded rows of a ragged batch are never written by the kernel
+        y = (torch.zeros if lens is not None else torch.empty)(
+            xbc.shape[0], heads * P, dtype=torch.float32, device=xbc.device)
+        _native().ssd_scan(xbc, dt_src, dt_col0, dt_bias, a_log, dskip,
+                           state, y, pos, lens, slots, T, heads, P, N, G)
+        return y
+    return ref.ssd_scan(xbc, dt_src, dt_col0, dt_bias, a_log, dskip, state,
+                        pos, T, heads, P, N, G, lens, slots)
+
+
+def delta_scan(src, r0: int, k0: int, v0: int, a0: int, wl, w0, ab, state,
+               pos, T: int, H: int, d: int, decay_scale: float,
+               unit_eps: float, lens=None, slots=None) -> torch.Tensor:
+    if src.is_cuda:
+        o = (torch.zeros if lens is not None else torch.empty)(
+            src.shape[0], H * d, dtype=torch.float32, device=src.device)
+        _native().delta_scan(src, r0, k0, v0, a0, wl, w0, ab, state, o, pos,
+                             lens, slots, T, H, d, decay_scale, unit_eps)
+        return o
+    return ref.delta_scan(src, r0, k0, v0, a0, wl, w0, ab, state, pos, T, H,
+                          d, decay_scale, unit_eps, lens, slots)
+
+
+def gated_group_rmsnorm(y, gate_src, gate_col0: int, w, groups: int,
+                        eps: float, gate_act: str, gate_first: bool,
+                        out_dtype: torch.dtype) -> torch.Tensor:
+    if y.is_cuda:
+        out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+        _native().gated_group_rmsnorm(y, gate_src, gate_col0, w, out, groups,
+                                      eps, gate_act == "silu", gate_first)
+        return out
+    return ref.gated_group_rmsnorm(y, gate_src, gate_col0, w, groups, eps,
+                                   gate_act, gate_first, out_dtype)
+
+
+_ACT_KINDS = {"relu_sq": 0, "tanh": 1}
+
+
+def act_slice(x, col0: int, n: int, kind: str) -> torch.Tensor:
+    if x.is_cuda:
+        y = torch.empty(x.shape[0], n, dtype=x.dtype, device=x.device)
+        _native().act_slice(x, col0, y, _ACT_KINDS[kind])
+        return y
+    return ref.act_slice(x, col0, n, kind)
+
+
+def gelu_gather_mul(z, table, tokens, col0: int) -> torch.Tensor:
+    if z.is_cuda:
+        y = torch.empty_like(z)
+        _native().gelu_gather_mul(z, table, tokens.reshape(-1), col0, y)
+        return y
+    return ref.gelu_gather_mul(z, table, tokens, col0)
+
+
+def resid_branches_rmsnorm(h, a, wa, b, wb, coef: float, f, wn, eps: float,
+                           out_dtype: torch.dtype, want_cast: bool = False):
+    """h (fp32, in place) += coef * (nrm(a, wa) + nrm(b, wb)) + f with
+    nrm(x, w) = x / rms(x) * w (or x when w is None); returns
+    (rms(h) * wn | None, h in out_dtype | None) — one kernel per boundary."""
+    if h.is_cuda:
+        assert h.dtype == torch.float32 and h.is_contiguous()
+        y = (torch.empty(h.shape, dtype=out_dtype, device=h.device)
+             if wn is not None else None)
+        xc = (torch.empty(h.shape, dtype=out_dtype, device=h.device)
+              if want_cast else None)
+        _native().resid_branches_rmsnorm(h, a, wa, b, wb, coef, f, wn, y, xc,
+                                         eps)
+        return y, xc
+    return ref.resid_branches_rmsnorm(h, a, wa, b, wb, coef, f, wn, eps,
+                                      out_dtype, want_cast)
+
+
+def clamped_glu(gu: torch.Tensor, alpha: float, limit: float) -> torch.Tensor:
+    if gu.is_cuda:
+        y = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype,
+                        device=gu.device)
+        _native().clamped_glu(gu, y, alpha, limit)
+        return y
+    return ref.clamped_glu(gu, alpha, limit)

@@ -12,6 +12,11 @@
 // j > i - window when window > 0). The sequence geometry lives in device
 // tensors, so a captured decode graph replays across steps.
 //
+// Pooled blocks (pool > 0, needs window > 0): beside the window's tokens a
+// query at position i sees entry c of the pooled caches pk/pv [Bc, Hkv, Sp, D]
+// (block means written by kv_pool_update) for every c < (i - window + 1) /
+// pool, in the same softmax and without a distance penalty.
+//
 // Two kernels:
 //  * attn_mod_rows<T>: flash-decode layout. One workgroup per (q tile, kv
 //    head, batch row): K/V chunks of 64 positions are staged through LDS once
@@ -92,9 +97,17 @@ struct ModParams {
   const float* r1;
   const float* r2;
   const float* sinks;
-  int T, Bc, Hq, Hkv, Smax, D, DV, QT, window;
+  const void* pk;      // pooled caches (same dtype as the cache) or null
+  const void* pv;
+  int T, Bc, Hq, Hkv, Smax, D, DV, QT, window, pool, Sp;
   float scale, softcap;
 };
+
+// pooled entries visible to a query at position i
+__device__ __forceinline__ int pool_count(int i, int window, int pool, int Sp) {
+  if (pool <= 0 || i < 0) return 0;
+  return min(Sp, max(0, (i - window + 1) / pool));
+}
 
 // transcendental flavours: fp32 models use the accurate library functions,
 // bf16 models the hardware approximations (error far below bf16 rounding)
@@ -130,8 +143,8 @@ __device__ __forceinline__ void stage16(float* dst, const float* src, bool on) {
 // robin and unnormalized (acc, m, l) go to `partial` [B, Hq, splits, DV+2].
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void attn_mod_rows(
-    const T* __restrict__ q, const T* __restrict__ kc,
-    const T* __restrict__ vc, T* __restrict__ out,
+    const T* __restrict__ q, const T* __restrict__ kc_tok,
+    const T* __restrict__ vc_tok, T* __restrict__ out,
     float* __restrict__ partial, const int splits, const ModParams P) {
   constexpr bool FAST = sizeof(T) == 2;
   constexpr bool PAIR = VEC && sizeof(T) == 2;
@@ -194,46 +207,62 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
   const int64_t kbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * D;
   const int64_t vbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * DV;
 
-  for (int s0 = (kv_begin & ~(kChunkR - 1)) + split * kChunkR; s0 < kv_end;
-       s0 += kChunkR * splits) {
-    const int valid = min(kChunkR, kv_end - s0);
+  // chunk list: pooled entries first, then the token range
+  const int np_max = pool_count(p0 + t0 + nt - 1, P.window, P.pool, P.Sp);
+  const int n_pc = (np_max + kChunkR - 1) / kChunkR;
+  const int tok0 = kv_begin & ~(kChunkR - 1);
+  const int n_tc = kv_end > tok0 ? (kv_end - tok0 + kChunkR - 1) / kChunkR : 0;
+  const int64_t pkbase = ((int64_t)slot * P.Hkv + hkv) * P.Sp * D;
+  const int64_t pvbase = ((int64_t)slot * P.Hkv + hkv) * P.Sp * DV;
+
+  for (int c = split; c < n_pc + n_tc; c += splits) {
+    const bool pooled = c < n_pc;
+    const int s0 = pooled ? c * kChunkR : tok0 + (c - n_pc) * kChunkR;
+    const int valid = min(kChunkR, (pooled ? np_max : kv_end) - s0);
+    const T* kc = pooled ? reinterpret_cast<const T*>(P.pk) + pkbase
+                         : kc_tok + kbase;
+    const T* vc = pooled ? reinterpret_cast<const T*>(P.pv) + pvbase
+                         : vc_tok + vbase;
     __syncthreads();          // previous chunk consumed (and q staged)
     if (VEC) {
       const int dk = D / EV, dvv = DV / EV;
       for (int idx = threadIdx.x; idx < kChunkR * dk; idx += blockDim.x) {
         const int r = idx / dk, e = (idx % dk) * EV;
-        stage16(&k_lds[r * PK + e], &kc[kbase + (int64_t)(s0 + r) * D + e],
+        stage16(&k_lds[r * PK + e], &kc[(int64_t)(s0 + r) * D + e],
                 r < valid);
       }
       for (int idx = threadIdx.x; idx < kChunkR * dvv; idx += blockDim.x) {
         const int r = idx / dvv, e = (idx % dvv) * EV;
-        stage16(&v_lds[r * PV + e], &vc[vbase + (int64_t)(s0 + r) * DV + e],
+        stage16(&v_lds[r * PV + e], &vc[(int64_t)(s0 + r) * DV + e],
                 r < valid);
       }
     } else {
       for (int idx = threadIdx.x; idx < kChunkR * D; idx += blockDim.x) {
         const int r = idx / D, e = idx % D;
         k_lds[r * PK + e] =
-            r < valid ? kc[kbase + (int64_t)(s0 + r) * D + e] : (T)0;
+            r < valid ? kc[(int64_t)(s0 + r) * D + e] : (T)0;
       }
       for (int idx = threadIdx.x; idx < kChunkR * DV; idx += blockDim.x) {
         const int r = idx / DV, e = idx % DV;
         v_lds[r * PV + e] =
-            r < valid ? vc[vbase + (int64_t)(s0 + r) * DV + e] : (T)0;
+            r < valid ? vc[(int64_t)(s0 + r) * DV + e] : (T)0;
       }
     }
     __syncthreads();
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
       const int i = qi[rr];
-      if (i < s0) continue;                 // wave-uniform: nothing visible
+      // entries of this chunk's source that row i may see: [0, lim)
+      const int lim = pooled ? pool_count(i, P.window, P.pool, P.Sp) : i + 1;
+      if (lim <= s0) continue;              // wave-uniform: nothing visible
       const int r = wid + 4 * rr;
       const int j = s0 + lane;
-      bool live = lane < valid && j <= i;
-      if (P.window > 0) live = live && (j > i - P.window);
+      bool live = lane < valid && j < lim;
+      if (!pooled && P.window > 0) live = live && (j > i - P.window);
       float s = dot_lds(&k_lds[lane * PK], &q_lds[r * PK], D) * tmp[rr];
       if (cap > 0.f) s = cap * m_tanh<FAST>(s * inv_cap);
-      if (P.r1) s -= r1[rr] * m_log1p<FAST>(r2[rr] * (float)max(i - j, 0));
+      if (P.r1 && !pooled)
+        s -= r1[rr] * m_log1p<FAST>(r2[rr] * (float)max(i - j, 0));
       if (!live) s = -INFINITY;
       const float mn = fmaxf(m[rr], wave_all_max(s));
       const float alpha = m_exp<FAST>(m[rr] - mn);
@@ -242,7 +271,7 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
       m[rr] = mn;
       p_lds[wid * kChunkR + lane] = p;
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // wave-local slab
-      const int vis = min(valid, i - s0 + 1);
+      const int vis = min(valid, lim - s0);
       const float* pw = &p_lds[wid * kChunkR];
       if (PAIR) {
         // lane owns dims (2*lane, 2*lane+1) + 128*jj
@@ -418,15 +447,30 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
   const float r1 = P.r1 ? P.r1[h] : 0.f, r2 = P.r1 ? P.r2[h] : 0.f;
 
   const int q_hi = min(tile0 + 63, n - 1);
-  const int s_end = min(P.Smax, p0 + q_hi + 1);
+  const short* kp_tok = kp;
+  const short* vp_tok = vp;
+
+  // phase 0: pooled entries (block means before the window); phase 1: tokens
+  for (int ph = P.pool > 0 ? 0 : 1; ph < 2; ++ph) {
+  const bool pooled = ph == 0;
+  const int Sdim = pooled ? P.Sp : P.Smax;
+  const int s_end = pooled ? pool_count(p0 + q_hi, P.window, P.pool, P.Sp)
+                           : min(P.Smax, p0 + q_hi + 1);
   int s_begin = 0;
-  if (P.window > 0) s_begin = max(0, p0 + tile0 - P.window + 1) & ~(ST - 1);
+  if (!pooled && P.window > 0)
+    s_begin = max(0, p0 + tile0 - P.window + 1) & ~(ST - 1);
+  kp = pooled ? reinterpret_cast<const short*>(P.pk) +
+                    ((int64_t)slot * P.Hkv + hk) * P.Sp * D
+              : kp_tok;
+  vp = pooled ? reinterpret_cast<const short*>(P.pv) +
+                    ((int64_t)slot * P.Hkv + hk) * P.Sp * DV
+              : vp_tok;
 
   for (int s0 = s_begin; s0 < s_end; s0 += ST) {
     __syncthreads();
     for (int idx = threadIdx.x; idx < ST * (DP / 8); idx += 256) {
       const int sr = idx / (DP / 8), dc = (idx % (DP / 8)) * 8;
-      const int sg = min(s0 + sr, P.Smax - 1);
+      const int sg = min(s0 + sr, Sdim - 1);
       short8 z;
 #pragma unroll
       for (int j = 0; j < 8; ++j) z.x[j] = 0;
@@ -435,7 +479,7 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
     }
     for (int idx = threadIdx.x; idx < ST * (DVP / 2); idx += 256) {
       const int sr = idx / (DVP / 2), dc = (idx % (DVP / 2)) * 2;
-      const int sg = min(s0 + sr, P.Smax - 1);
+      const int sg = min(s0 + sr, Sdim - 1);
       short v0 = 0, v1 = 0;
       if (dc < DV) {              // DV is even (multiple of 8)
         v0 = vp[(int64_t)sg * DV + dc];
@@ -463,9 +507,14 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
         const int i = p0 + qq;
         float val = sc[r] * sc_t;
         if (cap > 0.f) val = cap * fast_tanh(val * inv_cap);
-        if (P.r1) val -= r1 * __logf(1.f + r2 * (float)max(i - j, 0));
-        bool dead = (j > i) || (qq >= n) || (j >= P.Smax);
-        if (P.window > 0) dead |= (j <= i - P.window);
+        bool dead;
+        if (pooled) {
+          dead = (qq >= n) || (j >= pool_count(i, P.window, P.pool, P.Sp));
+        } else {
+          if (P.r1) val -= r1 * __logf(1.f + r2 * (float)max(i - j, 0));
+          dead = (j > i) || (qq >= n) || (j >= P.Smax);
+          if (P.window > 0) dead |= (j <= i - P.window);
+        }
         p_val[sub][r] = dead ? -INFINITY : val;
       }
     }
@@ -507,6 +556,7 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
                                                         0, 0);
     }
   }
+  }  // phases
 
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -553,7 +603,9 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
               double softcap, c10::optional<torch::Tensor> dist_r1,
               c10::optional<torch::Tensor> dist_r2,
               c10::optional<torch::Tensor> sinks, int64_t window,
-              c10::optional<torch::Tensor> partials, int64_t splits) {
+              c10::optional<torch::Tensor> partials, int64_t splits,
+              c10::optional<torch::Tensor> pool_k,
+              c10::optional<torch::Tensor> pool_v, int64_t pool) {
   DNET_CHECK(kcache.dim() == 4 && vcache.dim() == 4 &&
                  kcache.is_contiguous() && vcache.is_contiguous(), "cache");
   const int Bc = kcache.size(0), Hkv = kcache.size(1), Smax = kcache.size(2);
@@ -587,6 +639,25 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
   P.T = (int)T; P.Bc = Bc; P.Hq = Hq; P.Hkv = Hkv; P.Smax = Smax;
   P.D = D; P.DV = DV; P.window = (int)window;
   P.scale = (float)scale; P.softcap = (float)softcap;
+  P.pk = P.pv = nullptr;
+  P.pool = 0; P.Sp = 0;
+  if (pool > 0) {
+    DNET_CHECK(window > 0, "pooled blocks need a window");
+    DNET_CHECK(pool_k.has_value() && pool_v.has_value(), "pooled caches");
+    DNET_CHECK(pool_k->dim() == 4 && pool_k->is_contiguous() &&
+                   pool_v->dim() == 4 && pool_v->is_contiguous() &&
+                   pool_k->size(0) == Bc && pool_k->size(1) == Hkv &&
+                   pool_k->size(3) == D && pool_v->size(0) == Bc &&
+                   pool_v->size(1) == Hkv && pool_v->size(3) == DV &&
+                   pool_v->size(2) == pool_k->size(2) &&
+                   pool_k->scalar_type() == kcache.scalar_type() &&
+                   pool_v->scalar_type() == kcache.scalar_type(),
+               "pooled caches [Bc, Hkv, Sp, D|DV] in the cache dtype");
+    P.pk = pool_k->data_ptr();
+    P.pv = pool_v->data_ptr();
+    P.pool = (int)pool;
+    P.Sp = (int)pool_k->size(2);
+  }
   const int G = Hq / Hkv;
   const int GS = (G + kRowsMax - 1) / kRowsMax;
   P.QT = std::max(1, kRowsMax / std::min(G, kRowsMax));

@@ -78,7 +78,45 @@ void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
                    c10::optional<torch::Tensor> lens,
                    c10::optional<torch::Tensor> slots, double eps, int64_t nq,
                    int64_t nkv, int64_t d, int64_t dv, int64_t T,
-                   bool per_head);
+                   bool per_head, c10::optional<torch::Tensor> rot_freq);
+void resid_branches_rmsnorm(torch::Tensor h, torch::Tensor a,
+                            c10::optional<torch::Tensor> wa,
+                            c10::optional<torch::Tensor> b,
+                            c10::optional<torch::Tensor> wb, double coef,
+                            c10::optional<torch::Tensor> f,
+                            c10::optional<torch::Tensor> wn,
+                            c10::optional<torch::Tensor> y,
+                            c10::optional<torch::Tensor> xc, double eps);
+void gated_group_rmsnorm(torch::Tensor y, torch::Tensor gate_src,
+                         int64_t gate_col0, torch::Tensor w, torch::Tensor out,
+                         int64_t groups, double eps, bool gate_silu,
+                         bool gate_first);
+void act_slice(torch::Tensor x, int64_t col0, torch::Tensor y, int64_t kind);
+void gelu_gather_mul(torch::Tensor z, torch::Tensor table,
+                     torch::Tensor tokens, int64_t col0, torch::Tensor y);
+void clamped_glu(torch::Tensor gu, torch::Tensor y, double alpha,
+                 double limit);
+void kv_pool_update(torch::Tensor kcache, torch::Tensor vcache,
+                    torch::Tensor pool_k, torch::Tensor pool_v,
+                    torch::Tensor pos, c10::optional<torch::Tensor> lens,
+                    c10::optional<torch::Tensor> slots, int64_t T,
+                    int64_t pool);
+void causal_conv_silu(torch::Tensor x, int64_t col0, torch::Tensor w,
+                      torch::Tensor bias, torch::Tensor state, torch::Tensor y,
+                      torch::Tensor pos, c10::optional<torch::Tensor> lens,
+                      c10::optional<torch::Tensor> slots, int64_t T);
+void ssd_scan(torch::Tensor xbc, torch::Tensor dt_src, int64_t dt_col0,
+              torch::Tensor dt_bias, torch::Tensor a_log, torch::Tensor dskip,
+              torch::Tensor state, torch::Tensor y, torch::Tensor pos,
+              c10::optional<torch::Tensor> lens,
+              c10::optional<torch::Tensor> slots, int64_t T, int64_t heads,
+              int64_t P, int64_t N, int64_t G);
+void delta_scan(torch::Tensor src, int64_t r0, int64_t k0, int64_t v0,
+                int64_t a0, torch::Tensor wl, torch::Tensor w0,
+                torch::Tensor ab, torch::Tensor state, torch::Tensor o,
+                torch::Tensor pos, c10::optional<torch::Tensor> lens,
+                c10::optional<torch::Tensor> slots, int64_t T, int64_t H,
+                int64_t d, double decay_scale, double unit_eps);
 void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
               torch::Tensor pos, c10::optional<torch::Tensor> lens,
               c10::optional<torch::Tensor> slots, torch::Tensor out,
@@ -86,7 +124,9 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
               double softcap, c10::optional<torch::Tensor> dist_r1,
               c10::optional<torch::Tensor> dist_r2,
               c10::optional<torch::Tensor> sinks, int64_t window,
-              c10::optional<torch::Tensor> partials, int64_t splits);
+              c10::optional<torch::Tensor> partials, int64_t splits,
+              c10::optional<torch::Tensor> pool_k,
+              c10::optional<torch::Tensor> pool_v, int64_t pool);
 }  // namespace dnet
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -146,5 +186,23 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("qknorm_append", &dnet::qknorm_append,
         "q/k RMSNorm (whole projection or per head) + KV append");
   m.def("attn_mod", &dnet::attn_mod,
-        "score-modified causal attention (decode + ragged prefill)");
+        "score-modified causal attention (decode + ragged prefill), optional "
+        "window with pooled blocks");
+  m.def("resid_branches_rmsnorm", &dnet::resid_branches_rmsnorm,
+        "fp32 residual += normalized/plain branches, fused with the next "
+        "norm and a cast copy");
+  m.def("gated_group_rmsnorm", &dnet::gated_group_rmsnorm,
+        "grouped RMSNorm with a silu/sigmoid gate before or after");
+  m.def("act_slice", &dnet::act_slice,
+        "unary activation of a column range (relu^2, tanh)");
+  m.def("gelu_gather_mul", &dnet::gelu_gather_mul,
+        "gelu_tanh(z) * table[token, col0:col0+n]");
+  m.def("clamped_glu", &dnet::clamped_glu, "clamped GLU of [gate | up]");
+  m.def("kv_pool_update", &dnet::kv_pool_update,
+        "block means of the KV cache for the blocks a step completes");
+  m.def("causal_conv_silu", &dnet::causal_conv_silu,
+        "per-channel causal convolution + SiLU with a per-slot tail state");
+  m.def("ssd_scan", &dnet::ssd_scan,
+        "selective state-space recurrence (scalar decay per head)");
+  m.def("delta_scan", &dnet::delta_scan, "generalized delta-rule recurrence");
 }

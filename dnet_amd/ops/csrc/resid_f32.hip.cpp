@@ -7,7 +7,12 @@
 //                     layer boundary: residual update fused with the next norm)
 //   xielu             two-parameter squared / exponential activation
 //   qknorm_append     RMS-normalize q and k (whole projection or per head),
+//                     optionally rotate interleaved channel pairs by position,
 //                     write q, append k and v to the KV cache at pos[b]+t
+//   resid_branches_rmsnorm  h += coef*(nrm(a) + nrm(b)) + f with optional
+//                     RMS-normalized branches, next norm and a cast copy of h
+//   gated_group_rmsnorm     grouped RMSNorm with a silu / sigmoid gate
+//   act_slice, gelu_gather_mul, clamped_glu   small element-wise steps
 //
 // One workgroup per token row; statistics are block-reduced in fp32. "short"
 // stands for bf16 bits throughout.
@@ -157,7 +162,8 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
     const int* __restrict__ lens, const int* __restrict__ slots,
     const float eps, const int nq, const int nkv, const int d, const int dv,
     const int Tn, const int Bc, const int Hkv, const int Smax,
-    const bool per_head) {
+    const bool per_head, const float* __restrict__ rot_freq,
+    const int nrot) {
   __shared__ float red[8];
   const int64_t row = blockIdx.x;
   const int b = (int)(row / Tn);
@@ -218,13 +224,30 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
       const float r = 1.0f / sqrtf(ss / (float)d + eps);
-      if (isq) {
+      const float* wv = isq ? qw : kw;
+      T* dst = isq ? qo + hh * d
+                   : kc + kbase + (int64_t)(hh - nq) * Smax * d;
+      if (!isq && !keep) continue;
+      if (nrot > 0) {
+        // lanes own channel pairs (2i, 2i+1); pairs i < nrot turn by the
+        // angle position * rot_freq[i], computed and applied in fp32
+        for (int pr = lane; 2 * pr < d; pr += kWave) {
+          const int e0 = 2 * pr, e1 = e0 + 1;
+          float v0 = ldf<T>(hs + e0) * r * wv[e0];
+          float v1 = e1 < d ? ldf<T>(hs + e1) * r * wv[e1] : 0.f;
+          if (pr < nrot && e1 < d) {
+            float sn, cs;
+            sincosf((float)p * rot_freq[pr], &sn, &cs);
+            const float u0 = v0 * cs - v1 * sn;
+            v1 = v1 * cs + v0 * sn;
+            v0 = u0;
+          }
+          stf<T>(dst + e0, v0);
+          if (e1 < d) stf<T>(dst + e1, v1);
+        }
+      } else {
         for (int e = lane; e < d; e += kWave)
-          stf<T>(qo + hh * d + e, ldf<T>(hs + e) * r * qw[e]);
-      } else if (keep) {
-        for (int e = lane; e < d; e += kWave)
-          stf<T>(kc + kbase + (int64_t)(hh - nq) * Smax * d + e,
-                 ldf<T>(hs + e) * r * kw[e]);
+          stf<T>(dst + e, ldf<T>(hs + e) * r * wv[e]);
       }
     }
   }
@@ -234,6 +257,186 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
       stw<W, T>(vc + vbase + (int64_t)hk * Smax * dv + e,
                 ldw<W, T>(src + NQ + NK + i));
     }
+}
+
+
+// ---- branch sums, grouped gated norms, small element-wise steps ----------
+
+template <typename T>
+__device__ __forceinline__ float row_sumsq(const T* __restrict__ x, const int N,
+                                           float* red) {
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) {
+    const float v = ldf<T>(x + i);
+    ss += v * v;
+  }
+  return block_reduce_sum(ss, red);
+}
+
+// h += coef * (nrm(a, wa) + nrm(b, wb)) + f;  nrm(x, w) = x * rsqrt(mean(x^2)
+// + eps) * w, or x when w is null. Then y = rmsnorm(h) * wn (wn given) and
+// xc = h in the activation dtype (xc given). f may be fp32 or T.
+template <typename T, int W>
+__global__ __launch_bounds__(256) void resid_branches_kernel(
+    float* __restrict__ h, const T* __restrict__ a, const float* __restrict__ wa,
+    const T* __restrict__ b, const float* __restrict__ wb, const float coef,
+    const void* __restrict__ f, const bool f_f32, const float* __restrict__ wn,
+    T* __restrict__ y, T* __restrict__ xc, const int N, const float eps) {
+  __shared__ float red[8];
+  const int64_t row = blockIdx.x;
+  float* hr = h + row * N;
+  const T* ar = a + row * N;
+  const T* br = b ? b + row * N : nullptr;
+  float ra = 1.f, rb = 1.f;
+  if (wa) ra = 1.0f / sqrtf(row_sumsq<T>(ar, N, red) / (float)N + eps);
+  if (br && wb) rb = 1.0f / sqrtf(row_sumsq<T>(br, N, red) / (float)N + eps);
+  float ss = 0.f;
+  for (int i = threadIdx.x * W; i < N; i += blockDim.x * W) {
+    vecf<W> hv = ldw<W, float>(hr + i);
+    vecf<W> d = ldw<W, T>(ar + i);
+    if (wa) {
+      const vecf<W> g = ldw<W, float>(wa + i);
+#pragma unroll
+      for (int j = 0; j < W; ++j) d.v[j] = d.v[j] * ra * g.v[j];
+    }
+    if (br) {
+      vecf<W> e = ldw<W, T>(br + i);
+      if (wb) {
+        const vecf<W> g = ldw<W, float>(wb + i);
+#pragma unroll
+        for (int j = 0; j < W; ++j) e.v[j] = e.v[j] * rb * g.v[j];
+      }
+#pragma unroll
+      for (int j = 0; j < W; ++j) d.v[j] += e.v[j];
+    }
+#pragma unroll
+    for (int j = 0; j < W; ++j) d.v[j] *= coef;
+    if (f) {
+      const vecf<W> fv =
+          f_f32 ? ldw<W, float>(reinterpret_cast<const float*>(f) + row * N + i)
+                : ldw<W, T>(reinterpret_cast<const T*>(f) + row * N + i);
+#pragma unroll
+      for (int j = 0; j < W; ++j) d.v[j] += fv.v[j];
+    }
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      hv.v[j] += d.v[j];
+      ss += hv.v[j] * hv.v[j];
+    }
+    stw<W, float>(hr + i, hv);
+    if (xc) stw<W, T>(xc + row * N + i, hv);
+  }
+  if (!wn) return;                       // uniform
+  ss = block_reduce_sum(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)N + eps);
+  T* yr = y + row * N;
+  // each thread re-reads exactly the elements it wrote above
+  for (int i = threadIdx.x * W; i < N; i += blockDim.x * W) {
+    vecf<W> hv = ldw<W, float>(hr + i);
+    const vecf<W> g = ldw<W, float>(wn + i);
+#pragma unroll
+    for (int j = 0; j < W; ++j) hv.v[j] = hv.v[j] * r * g.v[j];
+    stw<W, T>(yr + i, hv);
+  }
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) {
+  return 1.0f / (1.0f + expf(-x));
+}
+
+// One wave per (row, group): out = rms_group(y [* gate]) * w [* gate], gate =
+// silu or sigmoid of columns [gcol0, gcol0+N) of gate_src (row stride gld).
+template <typename TG, typename TO>
+__global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(
+    const float* __restrict__ y, const TG* __restrict__ gate_src,
+    const int64_t gld, const int gcol0, const float* __restrict__ w,
+    TO* __restrict__ out, const int N, const int groups, const float eps,
+    const bool gate_silu, const bool gate_first) {
+  const int wid = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int64_t row = blockIdx.y;
+  const int grp = blockIdx.x * (blockDim.x / kWave) + wid;
+  if (grp >= groups) return;             // wave-uniform
+  const int gs = N / groups;
+  const float* yr = y + row * N + (int64_t)grp * gs;
+  const TG* gr = gate_src + row * gld + gcol0 + (int64_t)grp * gs;
+  float ss = 0.f;
+  for (int e = lane; e < gs; e += kWave) {
+    float v = yr[e];
+    if (gate_first) {
+      const float g = ldf<TG>(gr + e);
+      v *= gate_silu ? g * sigmoid_f(g) : sigmoid_f(g);
+    }
+    ss += v * v;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+  const float r = 1.0f / sqrtf(ss / (float)gs + eps);
+  TO* orow = out + row * N + (int64_t)grp * gs;
+  const float* wr = w + (int64_t)grp * gs;
+  for (int e = lane; e < gs; e += kWave) {
+    const float g = ldf<TG>(gr + e);
+    const float gv = gate_silu ? g * sigmoid_f(g) : sigmoid_f(g);
+    float v = yr[e];
+    if (gate_first) v *= gv;
+    v = v * r * wr[e];
+    if (!gate_first) v *= gv;
+    stf<TO>(orow + e, v);
+  }
+}
+
+// kind 0: max(z, 0)^2, kind 1: tanh(z); columns [col0, col0+n) of x (stride ld)
+template <typename T>
+__global__ __launch_bounds__(256) void act_slice_kernel(
+    const T* __restrict__ x, const int64_t ld, const int col0,
+    T* __restrict__ y, const int n, const int64_t total, const int kind) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = i / n;
+    const int c = (int)(i % n);
+    const float z = ldf<T>(x + row * ld + col0 + c);
+    float v;
+    if (kind == 0) {
+      const float t = fmaxf(z, 0.f);
+      v = t * t;
+    } else {
+      v = tanhf(z);
+    }
+    stf<T>(y + i, v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_gather_mul_kernel(
+    const T* __restrict__ z, const T* __restrict__ table, const int64_t tld,
+    const int64_t V, const int64_t* __restrict__ tokens, const int col0,
+    T* __restrict__ y, const int n, const int64_t total) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = i / n;
+    const int c = (int)(i % n);
+    int64_t tok = tokens[row];
+    tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);
+    const float v = ldf<T>(z + i);
+    const float g =
+        0.5f * v *
+        (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    stf<T>(y + i, g * ldf<T>(table + tok * tld + col0 + c));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void clamped_glu_kernel(
+    const T* __restrict__ gu, T* __restrict__ y, const int I,
+    const int64_t total, const float alpha, const float limit) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = i / I;
+    const int c = (int)(i % I);
+    const float g = fminf(ldf<T>(gu + row * 2 * I + c), limit);
+    const float u =
+        fminf(fmaxf(ldf<T>(gu + row * 2 * I + I + c), -limit), limit);
+    stf<T>(y + i, g * sigmoid_f(alpha * g) * (u + 1.0f));
+  }
 }
 
 static bool is_bf16(const torch::Tensor& t) {
@@ -347,8 +550,15 @@ void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
                    c10::optional<torch::Tensor> lens,
                    c10::optional<torch::Tensor> slots, double eps, int64_t nq,
                    int64_t nkv, int64_t d, int64_t dv, int64_t T,
-                   bool per_head) {
+                   bool per_head, c10::optional<torch::Tensor> rot_freq) {
   const int64_t M = qkv.size(0);
+  int nrot = 0;
+  if (rot_freq.has_value()) {
+    DNET_CHECK(per_head, "rotation comes with the per-head norm");
+    DNET_CHECK(is_f32(*rot_freq) && rot_freq->is_contiguous() &&
+                   rot_freq->numel() * 2 <= d, "rot_freq fp32 [<= d/2]");
+    nrot = (int)rot_freq->numel();
+  }
   DNET_CHECK(T > 0 && M % T == 0, "rows = B*T");
   const int64_t B = M / T;
   DNET_CHECK(qkv.is_contiguous() && qkv.size(1) == (nq + nkv) * d + nkv * dv,
@@ -379,12 +589,176 @@ void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
                      i32p(pos, B), i32p(lens, B), i32p(slots, B), (float)eps, \
                      (int)nq, (int)nkv, (int)d, (int)dv, (int)T, Bc, Hkv,     \
                      Smax,                                                   \
-                     per_head)
+                     per_head, nrot ? rot_freq->data_ptr<float>() : nullptr, \
+                     nrot)
   const bool v4 = d % 4 == 0 && dv % 4 == 0;
   if (is_bf16(qkv)) { if (v4) QA(short, 4); else QA(short, 1); }
   else if (is_f32(qkv)) { if (v4) QA(float, 4); else QA(float, 1); }
   else DNET_CHECK(false, "qknorm_append: dtype");
 #undef QA
+}
+
+void resid_branches_rmsnorm(torch::Tensor h, torch::Tensor a,
+                            c10::optional<torch::Tensor> wa,
+                            c10::optional<torch::Tensor> b,
+                            c10::optional<torch::Tensor> wb, double coef,
+                            c10::optional<torch::Tensor> f,
+                            c10::optional<torch::Tensor> wn,
+                            c10::optional<torch::Tensor> y,
+                            c10::optional<torch::Tensor> xc, double eps) {
+  const int N = h.size(-1);
+  const int64_t M = h.numel() / N;
+  DNET_CHECK(is_f32(h) && h.is_contiguous(), "h fp32 contiguous");
+  DNET_CHECK(a.is_contiguous() && a.numel() == h.numel() &&
+                 (is_bf16(a) || is_f32(a)), "a shape/dtype");
+  if (wa.has_value()) DNET_CHECK(wa->numel() == N, "wa fp32 [N]");
+  if (b.has_value())
+    DNET_CHECK(b->is_contiguous() && b->numel() == h.numel() &&
+                   b->scalar_type() == a.scalar_type(), "b shape/dtype");
+  if (wb.has_value()) DNET_CHECK(b.has_value() && wb->numel() == N, "wb");
+  bool f_f32 = false;
+  if (f.has_value()) {
+    DNET_CHECK(f->is_contiguous() && f->numel() == h.numel() &&
+                   (is_f32(*f) || f->scalar_type() == a.scalar_type()),
+               "f shape/dtype");
+    f_f32 = is_f32(*f);
+  }
+  DNET_CHECK(wn.has_value() == y.has_value(), "wn and y come together");
+  if (wn.has_value())
+    DNET_CHECK(wn->numel() == N && y->is_contiguous() &&
+                   y->numel() == h.numel() &&
+                   y->scalar_type() == a.scalar_type(), "y shape/dtype");
+  if (xc.has_value())
+    DNET_CHECK(xc->is_contiguous() && xc->numel() == h.numel() &&
+                   xc->scalar_type() == a.scalar_type(), "xc shape/dtype");
+  if (M == 0) return;
+  auto st = current_stream();
+#define RB(TT, WW)                                                           \
+  hipLaunchKernelGGL((resid_branches_kernel<TT, WW>), dim3(M), dim3(256), 0, \
+                     st, h.data_ptr<float>(), (const TT*)a.data_ptr(),       \
+                     f32p(wa),                                               \
+                     b.has_value() ? (const TT*)b->data_ptr() : nullptr,     \
+                     f32p(wb), (float)coef,                                  \
+                     f.has_value() ? (const void*)f->data_ptr() : nullptr,   \
+                     f_f32, f32p(wn),                                        \
+                     y.has_value() ? (TT*)y->data_ptr() : nullptr,           \
+                     xc.has_value() ? (TT*)xc->data_ptr() : nullptr, N,      \
+                     (float)eps)
+  const bool v4 = N % 4 == 0;
+  if (is_bf16(a)) { if (v4) RB(short, 4); else RB(short, 1); }
+  else { if (v4) RB(float, 4); else RB(float, 1); }
+#undef RB
+}
+
+void gated_group_rmsnorm(torch::Tensor y, torch::Tensor gate_src,
+                         int64_t gate_col0, torch::Tensor w, torch::Tensor out,
+                         int64_t groups, double eps, bool gate_silu,
+                         bool gate_first) {
+  DNET_CHECK(y.dim() == 2 && is_f32(y) && y.is_contiguous(), "y fp32 [M, N]");
+  const int64_t M = y.size(0);
+  const int N = y.size(1);
+  DNET_CHECK(groups > 0 && N % groups == 0, "groups divide N");
+  DNET_CHECK(gate_src.dim() == 2 && gate_src.is_contiguous() &&
+                 gate_src.size(0) == M && gate_col0 >= 0 &&
+                 gate_col0 + N <= gate_src.size(1), "gate columns");
+  DNET_CHECK(is_f32(w) && w.is_contiguous() && w.numel() == N, "w fp32 [N]");
+  DNET_CHECK(out.is_contiguous() && out.size(0) == M && out.size(1) == N,
+             "out [M, N]");
+  if (M == 0) return;
+  auto st = current_stream();
+  const dim3 grid((unsigned)((groups + 3) / 4), (unsigned)M);
+#define GG(TG, TO)                                                           \
+  hipLaunchKernelGGL((gated_group_rmsnorm_kernel<TG, TO>), grid, dim3(256),  \
+                     0, st, y.data_ptr<float>(),                             \
+                     (const TG*)gate_src.data_ptr(), gate_src.size(1),       \
+                     (int)gate_col0, w.data_ptr<float>(),                    \
+                     (TO*)out.data_ptr(), N, (int)groups, (float)eps,        \
+                     gate_silu, gate_first)
+  if (is_bf16(gate_src) && is_bf16(out)) GG(short, short);
+  else if (is_f32(gate_src) && is_f32(out)) GG(float, float);
+  else if (is_bf16(gate_src) && is_f32(out)) GG(short, float);
+  else if (is_f32(gate_src) && is_bf16(out)) GG(float, short);
+  else DNET_CHECK(false, "gated_group_rmsnorm: dtypes");
+#undef GG
+}
+
+static int ew_blocks(int64_t total) {
+  return (int)std::min<int64_t>((total + 255) / 256, 256 * 16);
+}
+
+void act_slice(torch::Tensor x, int64_t col0, torch::Tensor y, int64_t kind) {
+  DNET_CHECK(x.dim() == 2 && x.is_contiguous() && y.dim() == 2 &&
+                 y.is_contiguous() && y.size(0) == x.size(0) &&
+                 y.scalar_type() == x.scalar_type(), "act_slice: shapes");
+  const int n = y.size(1);
+  DNET_CHECK(col0 >= 0 && col0 + n <= x.size(1), "act_slice: columns");
+  DNET_CHECK(kind == 0 || kind == 1, "act_slice: kind");
+  const int64_t total = y.numel();
+  if (total == 0) return;
+  auto st = current_stream();
+  if (is_bf16(x))
+    hipLaunchKernelGGL((act_slice_kernel<short>), dim3(ew_blocks(total)),
+                       dim3(256), 0, st, (const short*)x.data_ptr(),
+                       x.size(1), (int)col0, (short*)y.data_ptr(), n, total,
+                       (int)kind);
+  else if (is_f32(x))
+    hipLaunchKernelGGL((act_slice_kernel<float>), dim3(ew_blocks(total)),
+                       dim3(256), 0, st, (const float*)x.data_ptr(),
+                       x.size(1), (int)col0, (float*)y.data_ptr(), n, total,
+                       (int)kind);
+  else DNET_CHECK(false, "act_slice: dtype");
+}
+
+void gelu_gather_mul(torch::Tensor z, torch::Tensor table,
+                     torch::Tensor tokens, int64_t col0, torch::Tensor y) {
+  DNET_CHECK(z.dim() == 2 && z.is_contiguous() && y.is_contiguous() &&
+                 y.numel() == z.numel() &&
+                 y.scalar_type() == z.scalar_type(), "gelu_gather_mul: z/y");
+  DNET_CHECK(table.dim() == 2 && table.is_contiguous() &&
+                 table.scalar_type() == z.scalar_type() && col0 >= 0 &&
+                 col0 + z.size(1) <= table.size(1), "table columns");
+  DNET_CHECK(tokens.scalar_type() == torch::kInt64 && tokens.is_contiguous() &&
+                 tokens.numel() == z.size(0), "tokens int64 [M]");
+  const int64_t total = z.numel();
+  if (total == 0) return;
+  auto st = current_stream();
+  if (is_bf16(z))
+    hipLaunchKernelGGL((gelu_gather_mul_kernel<short>),
+                       dim3(ew_blocks(total)), dim3(256), 0, st,
+                       (const short*)z.data_ptr(),
+                       (const short*)table.data_ptr(), table.size(1),
+                       table.size(0), tokens.data_ptr<int64_t>(), (int)col0,
+                       (short*)y.data_ptr(), (int)z.size(1), total);
+  else if (is_f32(z))
+    hipLaunchKernelGGL((gelu_gather_mul_kernel<float>),
+                       dim3(ew_blocks(total)), dim3(256), 0, st,
+                       (const float*)z.data_ptr(),
+                       (const float*)table.data_ptr(), table.size(1),
+                       table.size(0), tokens.data_ptr<int64_t>(), (int)col0,
+                       (float*)y.data_ptr(), (int)z.size(1), total);
+  else DNET_CHECK(false, "gelu_gather_mul: dtype");
+}
+
+void clamped_glu(torch::Tensor gu, torch::Tensor y, double alpha,
+                 double limit) {
+  DNET_CHECK(gu.dim() == 2 && gu.is_contiguous() && gu.size(1) % 2 == 0 &&
+                 y.is_contiguous() && y.size(0) == gu.size(0) &&
+                 y.size(1) * 2 == gu.size(1) &&
+                 y.scalar_type() == gu.scalar_type(), "clamped_glu: shapes");
+  const int64_t total = y.numel();
+  if (total == 0) return;
+  auto st = current_stream();
+  if (is_bf16(gu))
+    hipLaunchKernelGGL((clamped_glu_kernel<short>), dim3(ew_blocks(total)),
+                       dim3(256), 0, st, (const short*)gu.data_ptr(),
+                       (short*)y.data_ptr(), (int)y.size(1), total,
+                       (float)alpha, (float)limit);
+  else if (is_f32(gu))
+    hipLaunchKernelGGL((clamped_glu_kernel<float>), dim3(ew_blocks(total)),
+                       dim3(256), 0, st, (const float*)gu.data_ptr(),
+                       (float*)y.data_ptr(), (int)y.size(1), total,
+                       (float)alpha, (float)limit);
+  else DNET_CHECK(false, "clamped_glu: dtype");
 }
 
 }  // namespace dnet

@@ -519,15 +519,31 @@ def _row_index(B: int, T: int, pos, lens, slots, device):
     return p, ln, sl
 
 
+def rotate_pairs(x: torch.Tensor, ang: torch.Tensor) -> torch.Tensor:
+    """x [M, H, d] fp32, ang [M, n] fp32: pair (x[2i], x[2i+1]) -> (x[2i] cos
+    - x[2i+1] sin, x[2i+1] cos + x[2i] sin) for i < n (interleaved layout)."""
+    n = ang.shape[1]
+    c, s = torch.cos(ang).unsqueeze(1), torch.sin(ang).unsqueeze(1)
+    out = x.clone()
+    u, v = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
+    out[..., 0:2 * n:2] = u * c - v * s
+    out[..., 1:2 * n:2] = v * c + u * s
+    return out
+
+
 def qknorm_append(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor,
                   eps: float, nq: int, nkv: int, d: int, dv: int,
                   kcache: torch.Tensor, vcache: torch.Tensor,
                   pos: torch.Tensor, T: int, lens=None, slots=None,
-                  per_head: bool = False) -> torch.Tensor:
-    """RMS-normalize q and k (over the whole projection, or per head) and
-    append k, v to the cache. qkv [B*T, nq*d + nkv*d + nkv*dv]; token (b,t)
-    sits at position pos[b]+t of cache row slots[b]; tokens t >= lens[b]
-    are padding (not appended). Returns the normalized q [B*T, nq*d]."""
+                  per_head: bool = False,
+                  rot_freq: torch.Tensor | None = None) -> torch.Tensor:
+    """RMS-normalize q and k (over the whole projection, or per head),
+    optionally rotate them by position, and append k, v to the cache.
+    qkv [B*T, nq*d + nkv*d + nkv*dv]; token (b,t) sits at position pos[b]+t
+    of cache row slots[b]; tokens t >= lens[b] are padding (not appended).
+    ``rot_freq`` fp32 [n]: after the norm, channel pairs (2i, 2i+1), i < n,
+    of every head turn by the angle position * rot_freq[i] (fp32); channels
+    from 2n on pass unchanged. Returns the q rows [B*T, nq*d]."""
     M = qkv.shape[0]
     B = M // T
     q = qkv[:, :nq * d]
@@ -540,6 +556,20 @@ def qknorm_append(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor,
         qn = rmsnorm_rows(q, qw, eps, qkv.dtype)
         kn = rmsnorm_rows(k, kw, eps, qkv.dtype)
     p, ln, sl = _row_index(B, T, pos, lens, slots, qkv.device)
+    if rot_freq is not None:
+        # the rotation reads the fp32 normalized values (one rounding, at
+        # the end), like the fused kernel
+        if per_head:
+            qf = rmsnorm_rows(q.reshape(M, nq, d), qw, eps, torch.float32)
+            kf = rmsnorm_rows(k.reshape(M, nkv, d), kw, eps, torch.float32)
+        else:
+            qf = rmsnorm_rows(q, qw, eps, torch.float32).view(M, nq, d)
+            kf = rmsnorm_rows(k, kw, eps, torch.float32).view(M, nkv, d)
+        tpos = (p.view(B, 1) + torch.arange(T, device=qkv.device)
+                ).reshape(M).to(torch.float32)
+        ang = tpos.view(M, 1) * rot_freq.float().view(1, -1)
+        qn = rotate_pairs(qf, ang).reshape(M, -1).to(qkv.dtype)
+        kn = rotate_pairs(kf, ang).reshape(M, -1).to(qkv.dtype)
     for b in range(B):
         n = int(min(ln[b], T))
         if n <= 0:
@@ -555,12 +585,19 @@ def qknorm_append(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor,
 def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
              pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
              temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
-             sinks=None, window: int = 0) -> torch.Tensor:
+             sinks=None, window: int = 0, pool_k=None, pool_v=None,
+             pool: int = 0) -> torch.Tensor:
     """Causal attention against the cache with score modifiers, all in
     fp32: s = q.k * scale * temp[h]; s = cap*tanh(s/cap);
     s -= r1[h] * ln(1 + r2[h] * (i-j)); softmax whose denominator also
     holds exp(sink[h]). q [B*T, Hq*D] -> out [B*T, Hq*Dv]; query (b,t) is
-    at position pos[b]+t and sees keys j <= that (and > that - window)."""
+    at position pos[b]+t and sees keys j <= that (and > that - window).
+
+    With ``pool`` > 0 (needs a window): beside the window's tokens, query
+    i also sees entry c of the pooled caches ``pool_k`` / ``pool_v``
+    [Bc, Hkv, Sp, D|Dv] for every block c that ends at or before i - window
+    (c < (i - window + 1) // pool), in the same softmax; pooled entries take
+    no distance penalty."""
     Hkv, D = kcache.shape[1], kcache.shape[3]
     Dv = vcache.shape[3]
     M = q.shape[0]
@@ -594,6 +631,22 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
         if window and window > 0:
             dead = dead | (dist >= window)
         sc = sc.masked_fill(dead, float("-inf"))
+        nb = 0
+        if pool and window and window > 0:
+            nb = max(0, (S - 1 - window + 1) // pool)
+        if nb:
+            pk = pool_k[s, :, :nb].float()
+            pv = pool_v[s, :, :nb].float()
+            ps = torch.einsum("thgd,hsd->hgts", qq, pk) * scale
+            if temp is not None:
+                ps = ps * temp.float().view(Hkv, G, 1, 1)
+            if softcap and softcap > 0:
+                ps = softcap * torch.tanh(ps / softcap)
+            cnt = torch.div(i - window + 1, pool, rounding_mode="floor")
+            c = torch.arange(nb, device=q.device).view(1, nb)
+            ps = ps.masked_fill(c >= cnt, float("-inf"))
+            sc = torch.cat([sc, ps], dim=-1)
+            vv = torch.cat([vv, pv], dim=1)
         if sinks is not None:
             sk = sinks.float().view(Hkv, G, 1, 1).expand(Hkv, G, n, 1)
             pr = torch.softmax(torch.cat([sc, sk], dim=-1), dim=-1)[..., :-1]
@@ -602,3 +655,232 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
         o = torch.einsum("hgts,hsd->thgd", pr, vv)
         out[b * T:b * T + n] = o.reshape(n, Hq * Dv).to(q.dtype)
     return out
+
+
+# ---- pooled-block caches, short convolutions and linear recurrences ----
+# (sequence-state mixers: every state lives per cache row / slot, is taken as
+# zero at position 0 and is left untouched by padding tokens, so slots can be
+# reused without a reset and ragged batches equal each row alone)
+
+def kv_pool_update(kcache: torch.Tensor, vcache: torch.Tensor,
+                   pool_k: torch.Tensor, pool_v: torch.Tensor,
+                   pos: torch.Tensor, T: int, pool: int, lens=None,
+                   slots=None) -> None:
+    """Block means of the cache: for every block c of ``pool`` positions that
+    this step completes (its last position c*pool+pool-1 lies in
+    [pos[b], pos[b]+len)), pool_k[slot, :, c] = mean of the cached keys of the
+    block (fp32 sum of the values as stored, one rounding), same for v."""
+    B = pos.shape[0]
+    p, ln, sl = _row_index(B, T, pos, lens, slots, kcache.device)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        c0 = -(-(p0 - pool + 1) // pool)          # first block ending >= p0
+        c0 = max(c0, 0)
+        c = c0
+        while c * pool + pool - 1 < p0 + n and c < pool_k.shape[2]:
+            blk = slice(c * pool, (c + 1) * pool)
+            pool_k[s, :, c] = kcache[s, :, blk].float().mean(1).to(pool_k.dtype)
+            pool_v[s, :, c] = vcache[s, :, blk].float().mean(1).to(pool_v.dtype)
+            c += 1
+
+
+def causal_conv_silu(x: torch.Tensor, col0: int, w: torch.Tensor,
+                     bias: torch.Tensor, state: torch.Tensor,
+                     pos: torch.Tensor, T: int, lens=None,
+                     slots=None) -> torch.Tensor:
+    """Per-channel causal convolution + SiLU over columns [col0, col0+C) of
+    x [B*T, ld]. w fp32 [C, taps] (last tap = current token), bias fp32 [C];
+    ``state`` [Bc, taps-1, C] holds each slot's last taps-1 inputs (entry j =
+    position pos-(taps-1)+j; positions < 0 count as zero) and is advanced.
+    Returns fp32 [B*T, C] (padding rows zero)."""
+    C, taps = w.shape
+    M = x.shape[0]
+    B = M // T
+    xin = x[:, col0:col0 + C]
+    out = torch.zeros(M, C, dtype=torch.float32, device=x.device)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, x.device)
+    wf, bf = w.float(), bias.float()
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        hist = state[s].float().clone()                    # [taps-1, C]
+        for j in range(taps - 1):
+            if p0 - (taps - 1) + j < 0:
+                hist[j] = 0.0
+        seq = torch.cat([hist, xin[b * T:b * T + n].float()])
+        acc = bf.expand(n, C).clone()
+        for j in range(taps):
+            acc = acc + seq[j:j + n] * wf[:, j]
+        out[b * T:b * T + n] = acc * torch.sigmoid(acc)
+        if taps > 1:
+            state[s] = seq[n:].to(state.dtype)
+    return out
+
+
+def ssd_scan(xbc: torch.Tensor, dt_src: torch.Tensor, dt_col0: int,
+             dt_bias: torch.Tensor, a_log: torch.Tensor, dskip: torch.Tensor,
+             state: torch.Tensor, pos: torch.Tensor, T: int, heads: int,
+             P: int, N: int, G: int, lens=None, slots=None) -> torch.Tensor:
+    """Selective state-space recurrence with one scalar decay per head, all
+    fp32. xbc fp32 [B*T, heads*P + 2*G*N] = [x | B | C]; raw step sizes are
+    columns [dt_col0, dt_col0+heads) of dt_src. Per head h (group
+    g = h // (heads/G)), with dt = softplus(raw + dt_bias[h]):
+        S <- exp(-exp(a_log[h]) dt) S + dt B_g x_h^T      (S [N, P])
+        y_h = S^T C_g + dskip[h] x_h
+    ``state`` fp32 [Bc, heads, N, P] per slot: zero at position 0, advanced
+    by the real tokens. Returns y fp32 [B*T, heads*P]."""
+    M = xbc.shape[0]
+    B = M // T
+    inner = heads * P
+    y = torch.zeros(M, inner, dtype=torch.float32, device=xbc.device)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, xbc.device)
+    hg = torch.arange(heads, device=xbc.device) // (heads // G)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        S = state[s].float().clone() if p0 > 0 else \
+            torch.zeros(heads, N, P, dtype=torch.float32, device=xbc.device)
+        rows = slice(b * T, b * T + n)
+        xs = xbc[rows, :inner].float().view(n, heads, P)
+        Bm = xbc[rows, inner:inner + G * N].float().view(n, G, N)[:, hg]
+        Cm = xbc[rows, inner + G * N:].float().view(n, G, N)[:, hg]
+        dt = torch.nn.functional.softplus(
+            dt_src[rows, dt_col0:dt_col0 + heads].float() + dt_bias.float(),
+            threshold=30.0)
+        dec = torch.exp(-torch.exp(a_log.float()) * dt)        # [n, heads]
+        for t in range(n):
+            S = dec[t].view(heads, 1, 1) * S + dt[t].view(heads, 1, 1) * (
+                Bm[t].unsqueeze(-1) * xs[t].unsqueeze(1))
+            y[b * T + t] = ((S * Cm[t].unsqueeze(-1)).sum(1)
+                            + dskip.float().view(heads, 1) * xs[t]).reshape(-1)
+        state[s] = S
+    return y
+
+
+def delta_scan(src: torch.Tensor, r0: int, k0: int, v0: int, a0: int,
+               wl: torch.Tensor, w0: torch.Tensor, ab: torch.Tensor,
+               state: torch.Tensor, pos: torch.Tensor, T: int, H: int,
+               d: int, decay_scale: float, unit_eps: float, lens=None,
+               slots=None) -> torch.Tensor:
+    """Generalized delta rule, all fp32. r, k, v and the removal logits are
+    H*d-wide column ranges of src starting at r0, k0, v0, a0; wl [B*T, H*d]
+    holds the decay logits. Per head, with w = exp(-decay_scale *
+    sigmoid(wl + w0)), a = sigmoid(al + ab), u = k / sqrt(sum(k^2) +
+    unit_eps):
+        S <- diag(w) S - (a u)(u^T S) + k v^T     (both terms read the old S)
+        o = S^T r
+    ``state`` fp32 [Bc, H, d, d] per slot (key channel first): zero at
+    position 0. Returns o fp32 [B*T, H*d]."""
+    M = src.shape[0]
+    B = M // T
+    n_ = H * d
+    out = torch.zeros(M, n_, dtype=torch.float32, device=src.device)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, src.device)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        S = state[s].float().clone() if p0 > 0 else \
+            torch.zeros(H, d, d, dtype=torch.float32, device=src.device)
+        rows = slice(b * T, b * T + n)
+        col = lambda c0: src[rows, c0:c0 + n_].float().view(n, H, d)
+        r, k, v = col(r0), col(k0), col(v0)
+        a = torch.sigmoid(col(a0) + ab.float().view(H, d))
+        w = torch.exp(-decay_scale * torch.sigmoid(
+            wl[rows].float().view(n, H, d) + w0.float().view(H, d)))
+        u = k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)
+        for t in range(n):
+            uS = torch.einsum("hi,hij->hj", u[t], S)
+            S = w[t].unsqueeze(-1) * S \
+                - (a[t] * u[t]).unsqueeze(-1) * uS.unsqueeze(1) \
+                + k[t].unsqueeze(-1) * v[t].unsqueeze(1)
+            out[b * T + t] = torch.einsum("hij,hi->hj", S, r[t]).reshape(-1)
+        state[s] = S
+    return out
+
+
+def gated_group_rmsnorm(y: torch.Tensor, gate_src: torch.Tensor,
+                        gate_col0: int, w: torch.Tensor, groups: int,
+                        eps: float, gate_act: str, gate_first: bool,
+                        out_dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of y [M, N] in ``groups`` equal parts (each by its own root
+    mean square), times w [N], with a gate g = act(gate_src[:, gate_col0:
+    gate_col0+N]) (act = "silu" | "sigmoid") multiplied in before the norm
+    (gate_first) or after the weight. Statistics in fp32."""
+    M, N = y.shape
+    g = gate_src[:, gate_col0:gate_col0 + N].float()
+    g = g * torch.sigmoid(g) if gate_act == "silu" else torch.sigmoid(g)
+    v = y.float()
+    if gate_first:
+        v = v * g
+    v = v.view(M, groups, N // groups)
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    v = v.reshape(M, N) * w.float()
+    if not gate_first:
+        v = v * g
+    return v.to(out_dtype)
+
+
+def act_slice(x: torch.Tensor, col0: int, n: int, kind: str) -> torch.Tensor:
+    """Unary activation of columns [col0, col0+n) of x [M, ld], fp32 math:
+    "relu_sq" = max(z, 0)^2, "tanh"."""
+    z = x[:, col0:col0 + n].float()
+    if kind == "relu_sq":
+        z = torch.relu(z) ** 2
+    elif kind == "tanh":
+        z = torch.tanh(z)
+    else:
+        raise ValueError(kind)
+    return z.to(x.dtype)
+
+
+def gelu_gather_mul(z: torch.Tensor, table: torch.Tensor,
+                    tokens: torch.Tensor, col0: int) -> torch.Tensor:
+    """gelu_tanh(z[m, :]) * table[tokens[m], col0:col0+n] for z [M, n]."""
+    import math
+    zf = z.float()
+    g = 0.5 * zf * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi)
+                                     * (zf + 0.044715 * zf ** 3)))
+    e = table[tokens.reshape(-1).long(), col0:col0 + z.shape[1]].float()
+    return (g * e).to(z.dtype)
+
+
+def resid_branches_rmsnorm(h: torch.Tensor, a: torch.Tensor, wa, b, wb,
+                           coef: float, f, wn, eps: float,
+                           out_dtype: torch.dtype, want_cast: bool):
+    """h (fp32, in place) += coef * (nrm(a, wa) + nrm(b, wb)) + f, where
+    nrm(x, w) = x / rms(x) * w when w is given and x itself otherwise (b and
+    f optional). Returns (rms(h) * wn or None, h cast to out_dtype or
+    None)."""
+    def nrm(x, w):
+        xf = x.float()
+        if w is None:
+            return xf
+        return xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) \
+            * w.float()
+    d = nrm(a, wa)
+    if b is not None:
+        d = d + nrm(b, wb)
+    d = d * coef
+    if f is not None:
+        d = d + f.float()
+    h.add_(d)
+    y = rmsnorm_rows(h, wn, eps, out_dtype) if wn is not None else None
+    return y, (h.to(out_dtype) if want_cast else None)
+
+
+def clamped_glu(gu: torch.Tensor, alpha: float, limit: float) -> torch.Tensor:
+    """gu [M, 2I] = [gate | up]: g = min(gate, limit), u = clamp(up,
+    -limit, limit); y = g * sigmoid(alpha * g) * (u + 1), fp32 math."""
+    i = gu.shape[-1] // 2
+    g = gu[..., :i].float().clamp(max=limit)
+    u = gu[..., i:].float().clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)

@@ -122,6 +122,12 @@ class RingExecutor:
                              self.is_last, smax=smax, tp_rank=self.tp_rank,
                              tp_size=tp, tp_group=stage_group)
         self.model.kv_bits = kv_bits
+        if getattr(self.model, "needs_tokens", False) and self.stages > 1:
+            # the ring hops carry the residual only; layers that read the
+            # token ids again need them on every stage
+            raise NotImplementedError(
+                f"{cfg.model_type}: pipeline stages are not implemented "
+                "(every layer reads the token ids)")
         if init_weights:
             self.model.init_random(seed)
         self.weight_cache = None
@@ -563,11 +569,17 @@ class RingExecutor:
 
     t_replay = 0.0   # cumulative; slot-tick profiling
 
-    def slot_step_compute(self, mb: int = 0) -> None:
+    def slot_step_compute(self, mb: int = 0, park=None) -> None:
         """One decode step over the whole slot batch, including the ring
-        hops — no sampling (the caller samples on the last stage)."""
+        hops — no sampling (the caller samples on the last stage).
+        ``park`` (bool [slots], device): rows that sit this step out; models
+        with per-slot recurrent state leave those rows' state untouched
+        (the mask is copied into the cache's static ``idle`` buffer, which
+        the captured step reads)."""
         import time as _t
         _t0 = _t.perf_counter()
+        if park is not None:
+            self.kvs[mb].idle.copy_(park)
         self._slot_step_compute_inner(mb)
         self.t_replay += _t.perf_counter() - _t0
 

@@ -814,7 +814,7 @@ class ShardRuntime:
         broadcast, identical slot-state update on every rank."""
         ex = self.executor
         rs = self._row_sampler
-        ex.slot_step_compute()
+        ex.slot_step_compute(park=self._park_dev)
         if ex.is_last:
             toks_t = self._row_sampler.sample(ex.logits_buf[0].float())
             ex.tokbuf[0].copy_(toks_t)
@@ -849,7 +849,7 @@ class ShardRuntime:
             self._launch_evs = (torch.cuda.Event(enable_timing=True),
                                 torch.cuda.Event(enable_timing=True))
             self._launch_evs[0].record()
-        ex.slot_step_compute()
+        ex.slot_step_compute(park=self._park_dev)
         t0 = time.perf_counter()
         toks_t = self._row_sampler.sample(ex.logits_buf[0].float())
         self._t_sample += time.perf_counter() - t0
