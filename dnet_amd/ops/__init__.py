@@ -74,6 +74,15 @@ def _get_scratch(device) -> torch.Tensor:
     return _scratch[key]
 
 
+def scratch_clean(device) -> None:
+    """Zero what plain split-k combines left in the scratch (a fill kernel,
+    launched only when something is dirty). The decode-graph executor calls
+    it before a replay and as the last node of every captured step, so
+    eager small-M GEMMs (prefill logits) and graph replays can alternate."""
+    if torch.device(device).type == "cuda" and str(device) in _scratch:
+        _native().scratch_clean(_scratch[str(device)])
+
+
 def gemv_bf16(x: torch.Tensor, w: torch.Tensor,
               bias: torch.Tensor | None = None) -> torch.Tensor:
     if x.is_cuda:

@@ -653,6 +653,43 @@ __global__ void f32_to_bf16_bias_kernel(const float* __restrict__ in,
 // own M*N region and corrupt the next bigger user.
 static int64_t g_scratch_dirty_elems = 0;
 
+// Scratch clears are a small fill kernel, never a memset node: the clear may
+// be recorded into a captured decode graph.
+__global__ __launch_bounds__(256) void zero_fill_kernel(float* __restrict__ p,
+                                                        const int64_t n) {
+  const int64_t n4 = (n + 3) / 4;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    if (4 * i + 3 < n) {
+      reinterpret_cast<float4*>(p)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+      for (int64_t j = 4 * i; j < n; ++j) p[j] = 0.f;
+    }
+  }
+}
+
+static void zero_fill(float* p, int64_t elems, hipStream_t stream) {
+  if (elems <= 0) return;
+  const int64_t n4 = (elems + 3) / 4;
+  const int grid = (int)std::min<int64_t>((n4 + 255) / 256, 2048);
+  hipLaunchKernelGGL(zero_fill_kernel, dim3(grid), dim3(256), 0, stream, p,
+                     elems);
+}
+
+// Zero whatever plain combines left behind and forget it. A captured step
+// starts from a clean scratch and ends with this call, so replays and eager
+// launches can alternate: the host-side count above describes the device
+// state at every boundary between them.
+void scratch_clean(torch::Tensor scratch) {
+  if (g_scratch_dirty_elems <= 0) return;
+  DNET_CHECK(scratch.scalar_type() == torch::kFloat32 &&
+                 scratch.is_contiguous(), "scratch fp32");
+  zero_fill(scratch.data_ptr<float>(),
+            std::min<int64_t>(g_scratch_dirty_elems, scratch.numel()),
+            current_stream());
+  g_scratch_dirty_elems = 0;
+}
+
 static int pick_splitk(int64_t N, int64_t K, int64_t M, int64_t scratch_elems,
                        int min_pairs, int g_align) {
   // Target ~1024 blocks (~4 blocks / 16 waves per CU) so HBM latency is
@@ -720,7 +757,7 @@ static bool launch_m16(torch::Tensor x, torch::Tensor w,
     if (g_scratch_dirty_elems > 0) {
       const int64_t span = std::max<int64_t>(g_scratch_dirty_elems,
                                              (int64_t)M * N);
-      DNET_CHECK_HIP(hipMemsetAsync(fp, 0, sizeof(float) * span, stream));
+      zero_fill(fp, std::min<int64_t>(span, scratch->numel()), stream);
       g_scratch_dirty_elems = 0;
     }
   }

@@ -22,6 +22,7 @@ from typing import Optional
 import torch
 import torch.distributed as dist
 
+from .. import ops
 from ..core.sampler import DecodingConfig, Sampler
 from ..models import KVCache, ModelConfig, get_ring_model
 from .comm import Ring
@@ -233,8 +234,26 @@ class RingExecutor:
         if self.is_last and r == self.rounds - 1:
             self.logits_buf[mb].copy_(
                 self.model.normalize_project(self.hbuf[mb]))
+        # leave the split-k scratch clean: a captured step must end in the
+        # state it assumes at its start
+        ops.scratch_clean(self.device)
 
     def _capture_graphs(self):
+        # warm-up runs execute the step body for real: with every row marked
+        # idle they append nothing and leave per-slot recurrent state alone
+        # (models without such state ignore the mask; their dummy appends
+        # land on rows that real steps rewrite)
+        saved_idle = [kv.idle.clone() for kv in self.kvs]
+        for kv in self.kvs:
+            kv.idle.fill_(True)
+        try:
+            self._capture_graphs_inner()
+        finally:
+            for kv, m in zip(self.kvs, saved_idle):
+                kv.idle.copy_(m)
+
+    def _capture_graphs_inner(self):
+        ops.scratch_clean(self.device)
         pool = torch.cuda.graph_pool_handle()
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
@@ -277,6 +296,7 @@ class RingExecutor:
                 self.use_graphs = False
                 self._graphs = {}
         if self.use_graphs:
+            ops.scratch_clean(self.device)   # eager GEMMs since the last replay
             f = self._graph_flip[(mb, r)]
             self._graphs[(mb, r)][f].replay()
             self._graph_flip[(mb, r)] = f ^ 1
