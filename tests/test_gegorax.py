@@ -1,0 +1,749 @@
+"""Gegorax in the framework against the plain oracle (tests/gegorax_oracle.py).
+
+Every test builds its own small configuration and random checkpoint, runs it
+through the framework's ops / model / cache / executor (and, for generation,
+the shard runtime's slot scheduler and the trace replay CLI) and compares with
+the oracle, which is written from the equations in double precision and shares
+no code with dnet_amd. Tests run on the CPU reference-op path and, marked
+``gpu``, on the HIP kernels.
+"""
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+import dnet_amd.ops as ops
+import gegorax_oracle as O
+from dnet_amd.models import ModelConfig
+from dnet_amd.parallel.ring import RingExecutor
+
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
+F64 = torch.float64
+
+
+# ---------- small random checkpoints ----------
+
+def par(heads=4, kv=2, dim=16, vdim=8, size=9, pool=3, rot=12, base=500.0,
+        sh=3, svd=8, state=8, groups=1, ng=1, conv=3, scale=None):
+    left = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim,
+            "scale": scale if scale is not None else dim ** -0.5}
+    if size:
+        left["mask"] = {"size": size}
+        if pool:
+            left["mask"]["pool"] = pool
+    if rot:
+        left["rot"] = {"dims": rot, "base": base}
+    return {"left": left,
+            "right": {"conv": conv, "groups": groups, "heads": sh,
+                      "norm_groups": ng, "state": state, "vdim": svd}}
+
+
+def delta(heads=2, dim=8):
+    return {"heads": heads, "dim": dim}
+
+
+def moe(experts=5, top=2, ff=12, limit=1.2, shared=10, slimit=0.8):
+    m = {"kind": "moe", "router": {"experts": experts, "top": top},
+         "expert": {"ff": ff, "limit": limit}}
+    if shared:
+        m["shared"] = {"ff": shared, "limit": slimit}
+    return m
+
+
+def dense(ff=40):
+    return {"kind": "dense", "ff": ff}
+
+
+def make_cfg(layers, width=40, vocab=83, eps=1e-5, side=6):
+    import copy
+    cfg = {"architecture": "Gegorax", "vocab": vocab, "width": width,
+           "norm": {"eps": eps},
+           "layers": [{"type": "parallel" if "left" in m else "general_delta",
+                       "mixer": copy.deepcopy(m), "mlp": copy.deepcopy(ff)}
+                      for m, ff in layers]}
+    if side:
+        cfg["token_side"] = {"dim": side}
+    return cfg
+
+
+BASE = [(par(), dense()), (delta(), moe()), (delta(2, 16), dense(24)),
+        (par(heads=2, kv=2, size=6, pool=2, rot=16, sh=4, svd=4, state=16,
+             groups=2, ng=2, conv=4), moe(experts=4, top=1, shared=0))]
+
+
+def make_weights(cfg, seed=0, rank=4, dtype="float32"):
+    """Random checkpoint. For bfloat16 runs the routers get a small input
+    gain and widely spread biases: which experts a token takes then does not
+    hang on a near-tie that rounding could flip (input-dependent routing is
+    compared in float32, and at the mechanism level on identical inputs)."""
+    g = torch.Generator().manual_seed(seed)
+    steady = dtype == "bfloat16"
+    W, V = cfg["width"], cfg["vocab"]
+
+    def rn(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16)
+
+    def ru(n, lo, hi):
+        return (torch.rand(n, generator=g) * (hi - lo) + lo).to(torch.bfloat16)
+
+    def lin(o, i, gain=1.0):
+        return rn(o, i, std=gain * i ** -0.5)
+
+    sd = {"embed": rn(V, W), "final.norm": 1 + rn(W, std=0.2),
+          "head": lin(V, W)}
+    side = (cfg.get("token_side") or {}).get("dim", 0)
+    if side:
+        sd["side.embed"] = rn(V, side * len(cfg["layers"]))
+    for i, spec in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        m = spec["mixer"]
+        sd[p + "norm1"] = 1 + rn(W, std=0.2)
+        if spec["type"] == "parallel":
+            lf, rt = m["left"], m["right"]
+            H, G, d, dv = lf["heads"], lf["kv_heads"], lf["dim"], lf["vdim"]
+            inner = rt["heads"] * rt["vdim"]
+            C = inner + 2 * rt["groups"] * rt["state"]
+            sd.update({
+                p + "mix.left.q": lin(H * d, W, 2.0),
+                p + "mix.left.k": lin(G * d, W, 2.0),
+                p + "mix.left.v": lin(G * dv, W),
+                p + "mix.left.q.norm": 1 + rn(d, std=0.3),
+                p + "mix.left.k.norm": 1 + rn(d, std=0.3),
+                p + "mix.left.o": lin(W, H * dv),
+                p + "mix.right.in": lin(2 * inner + 2 * rt["groups"]
+                                        * rt["state"] + rt["heads"], W),
+                p + "mix.right.conv": rn(C, rt["conv"], std=0.6),
+                p + "mix.right.conv.b": rn(C, std=0.2),
+                p + "mix.right.dt_bias": ru(rt["heads"], -2.0, 0.5),
+                p + "mix.right.A_log": ru(rt["heads"], -2.0, 1.0),
+                p + "mix.right.D": rn(rt["heads"]),
+                p + "mix.right.norm": 1 + rn(inner, std=0.3),
+                p + "mix.right.o": lin(W, inner),
+                p + "mix.left.out": 1 + rn(W, std=0.3),
+                p + "mix.right.out": 1 + rn(W, std=0.3)})
+        else:
+            n = m["heads"] * m["dim"]
+            for name in ("r", "k", "v", "g", "a"):
+                sd[p + "mix." + name] = lin(n, W)
+            sd.update({p + "mix.a.b": rn(n, std=0.5),
+                       p + "mix.w1": lin(rank, W),
+                       p + "mix.w2": lin(n, rank, 2.0),
+                       p + "mix.w0": rn(n),
+                       p + "mix.norm": 1 + rn(n, std=0.3),
+                       p + "mix.o": lin(W, n)})
+        ff = spec["mlp"]
+        if ff is not None and ff["kind"] == "dense":
+            sd[p + "mlp.up"] = lin(ff["ff"], W)
+            sd[p + "mlp.down"] = lin(W, ff["ff"])
+        elif ff is not None:
+            E = ff["router"]["experts"]
+            sd[p + "mlp.router"] = lin(E, W, 0.05 if steady else 3.0)
+            sd[p + "mlp.router.b"] = (
+                (torch.randperm(E, generator=g) * 1.5).to(torch.bfloat16)
+                if steady else rn(E, std=0.5))
+            names = [(f"e{e}", ff["expert"]["ff"]) for e in range(E)]
+            if ff.get("shared"):
+                names.append(("shared", ff["shared"]["ff"]))
+            for name, sz in names:
+                sd[p + f"mlp.{name}.gate"] = lin(sz, W, 2.0)
+                sd[p + f"mlp.{name}.up"] = lin(sz, W, 2.0)
+                sd[p + f"mlp.{name}.down"] = lin(W, sz)
+        if side:
+            sd[p + "side.gate"] = lin(side, W)
+            sd[p + "side.proj"] = lin(W, side)
+            sd[p + "side.norm"] = ru(W, 0.3, 1.2)
+    return sd
+
+
+def executor(cfg, sd, device, dtype="float32", slots=4, smax=160, **kw):
+    mc = ModelConfig.from_hf(cfg)
+    mc.compute_dtype = dtype
+    ex = RingExecutor(mc, 0, 1, device, mb_count=1, mb_size=slots, smax=smax,
+                      init_weights=False, use_graphs=False, **kw)
+    ex.model.load_state_dict(sd)
+    return ex
+
+
+def tokens(n, vocab, seed):
+    return torch.randint(0, vocab, (n,),
+                         generator=torch.Generator().manual_seed(seed))
+
+
+def close(got, want, dtype="float32"):
+    got, want = got.detach().cpu().to(F64), want.to(F64)
+    scale = float(want.pow(2).mean().sqrt())
+    # float32 is the sharp comparison; in bfloat16 single positions of these
+    # tiny models amplify rounding noise (norms of small vectors), so the
+    # bound is on the root mean square with a loose cap on any one entry
+    tol = 2e-4 if dtype == "float32" else 2.5e-1
+    err = float((got - want).abs().max())
+    assert err <= tol * scale, f"max err {err:.3g} vs scale {scale:.3g}"
+    rms = float((got - want).pow(2).mean().sqrt())
+    assert rms <= 0.3 * tol * scale, f"rms err {rms:.3g} vs {scale:.3g}"
+
+
+def decode_steps(ex, slot_tokens):
+    """One slot-batch decode step: {slot: token}; other rows sit it out.
+    Returns the logits [slots, V]."""
+    tb = ex.tokbuf[0].cpu()
+    for s, t in slot_tokens.items():
+        tb[s] = int(t)
+    ex.tokbuf[0].copy_(tb)
+    idle = torch.ones(ex.mb_size, dtype=torch.bool)
+    idle[list(slot_tokens)] = False
+    idle = idle.to(ex.device)
+    ex.slot_step_compute(park=idle)
+    lg = ex.logits_buf[0].float().cpu().clone()
+    pos = ex.kvs[0].pos
+    pos.add_((~idle).to(pos.dtype))
+    return lg
+
+
+def oracle(toks, cfg, sd):
+    return O.forward(toks.tolist(), cfg, sd)
+
+
+# ---------- configuration ----------
+
+def test_config_and_registry():
+    from dnet_amd.models import GegoraxRingModel, get_ring_model
+    cfg = make_cfg(BASE)
+    mc = ModelConfig.from_hf(cfg)
+    assert mc.model_type == "gegorax" and mc.num_layers == 4
+    assert mc.token_side_dim == 6 and mc.num_experts == 5
+    assert get_ring_model("gegorax") is GegoraxRingModel
+    bad = make_cfg(BASE)
+    bad["layers"][0]["type"] = "conv"
+    with pytest.raises(ValueError):
+        ModelConfig.from_hf(bad)
+    bad = make_cfg(BASE)
+    bad["layers"][1]["mlp"]["kind"] = "glu"
+    with pytest.raises(ValueError):
+        ModelConfig.from_hf(bad)
+    bad = make_cfg([(par(size=0, pool=0), None)])
+    bad["layers"][0]["mixer"]["left"]["mask"] = {"pool": 4}
+    with pytest.raises(ValueError):
+        ModelConfig.from_hf(bad)
+
+
+# ---------- mechanisms alone ----------
+
+def _cache_attention(device, dt, q, k, v, scale, size, pool, T0):
+    """q [T,H,d], k [T,G,d], v [T,G,dv] as cached values: the first T0
+    positions arrive as one prompt portion, the rest token by token."""
+    T, H, d = q.shape
+    G, dv = k.shape[1], v.shape[2]
+    S = 64
+    kc = torch.zeros(2, G, S, d, dtype=dt, device=device)
+    vc = torch.zeros(2, G, S, dv, dtype=dt, device=device)
+    nb = S // max(pool, 1) + 1
+    pk = torch.zeros(2, G, nb, d, dtype=dt, device=device)
+    pv = torch.zeros(2, G, nb, dv, dtype=dt, device=device)
+    slot = torch.tensor([1], dtype=torch.int32, device=device)
+    outs = []
+    steps = [(0, T0)] + [(t, 1) for t in range(T0, T)]
+    for p0, n in steps:
+        kc[1, :, p0:p0 + n] = k[p0:p0 + n].transpose(0, 1).to(dt).to(device)
+        vc[1, :, p0:p0 + n] = v[p0:p0 + n].transpose(0, 1).to(dt).to(device)
+        pos = torch.tensor([p0], dtype=torch.int32, device=device)
+        ln = torch.tensor([n], dtype=torch.int32, device=device)
+        if pool:
+            ops.kv_pool_update(kc, vc, pk, pv, pos, n, pool, ln, slot)
+        qq = q[p0:p0 + n].reshape(n, H * d).to(dt).to(device).contiguous()
+        outs.append(ops.attn_mod(qq, kc, vc, pos, n, scale, ln, slot,
+                                 window=size, pool_k=pk if pool else None,
+                                 pool_v=pv if pool else None, pool=pool))
+    return torch.cat(outs).view(T, H, dv)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("size,pool", [(7, 3), (5, 1), (8, 4), (6, 0)])
+def test_window_edges_and_pooled_blocks(device, size, pool):
+    """One key at a time is made to dominate its score (query and key share
+    a large component): the key just inside the window, the one just
+    outside it, one deep in a pooled block, and a block that is just
+    complete / not yet complete behind the window. A window or block that
+    is one position off moves the output by the whole value."""
+    torch.manual_seed(size * 10 + pool)
+    T, H, G, d, dv = 40, 2, 1, 8, 4
+    q = torch.randn(T, H, d, dtype=F64)
+    k = torch.randn(T, G, d, dtype=F64) * 0.3
+    v = torch.randn(T, G, dv, dtype=F64)
+    spike = torch.zeros(d, dtype=F64)
+    spike[0] = 6.0
+    for i, j in ((30, 30 - size + 1), (33, 33 - size), (36, 2),
+                 (38, 38 - size - (pool or 1) + 1), (39, 39 - size - 1)):
+        q[i] += spike
+        k[j] += spike
+    want = O.window_pool_attention(q, k, v, 0.5, size, pool)
+    for T0 in (T, 12):         # whole prompt; short prompt + decoding
+        got = _cache_attention(device, torch.float32, q, k, v, 0.5, size,
+                               pool, T0)
+        close(got, want)
+    got = _cache_attention(device, torch.bfloat16, q, k, v, 0.5, size, pool,
+                           20)
+    kb, vb = k.to(torch.bfloat16).to(F64), v.to(torch.bfloat16).to(F64)
+    close(got, O.window_pool_attention(q.to(torch.bfloat16).to(F64), kb, vb,
+                                       0.5, size, pool), "bfloat16")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_rotation_and_qk_norm(device):
+    """Per-head norm, then interleaved pairs of the first rot.dims channels
+    turn by position * base^(-2i/dims); the rest pass; v is untouched."""
+    torch.manual_seed(3)
+    nq, nkv, d, dv, T = 3, 1, 10, 6, 7
+    dims, base, eps = 6, 50.0, 1e-5
+    qkv = torch.randn(T, (nq + nkv) * d + nkv * dv)
+    qw, kw = torch.randn(d), torch.randn(d)
+    freq = torch.tensor([base ** (-2.0 * i / dims) for i in range(dims // 2)],
+                        dtype=torch.float32)
+    kc = torch.zeros(1, nkv, 64, d, device=device)
+    vc = torch.zeros(1, nkv, 64, dv, device=device)
+    p0 = 41
+    pos = torch.tensor([p0], dtype=torch.int32, device=device)
+    q = ops.qknorm_append(qkv.to(device), qw.to(device), kw.to(device), eps,
+                          nq, nkv, d, dv, kc, vc, pos, T, per_head=True,
+                          rot_freq=freq.to(device))
+    x = qkv.to(F64)
+    positions = torch.arange(p0, p0 + T)
+    rot = {"dims": dims, "base": base}
+    qo = O.rotate(O.rms(x[:, :nq * d].view(T, nq, d), eps) * qw.to(F64),
+                  positions, rot)
+    ko = O.rotate(O.rms(x[:, nq * d:(nq + nkv) * d].view(T, nkv, d), eps)
+                  * kw.to(F64), positions, rot)
+    close(q.view(T, nq, d), qo)
+    close(kc[0, :, p0:p0 + T].transpose(0, 1), ko)
+    close(vc[0, :, p0:p0 + T].transpose(0, 1),
+          x[:, (nq + nkv) * d:].view(T, nkv, dv))
+    assert float(kc[0, :, :p0].abs().max()) == 0.0
+
+
+def _one_layer(device, dtype, mixer, ff, side=0, seed=1, T=21, width=24):
+    cfg = make_cfg([(mixer, ff)], width=width, vocab=37, side=side)
+    sd = make_weights(cfg, seed, dtype=dtype)
+    ex = executor(cfg, sd, device, dtype, slots=2, smax=64)
+    toks = tokens(T, 37, seed)
+    got = ex.prefill_slots([1], [toks], want=[list(range(T))])[0]
+    close(got, oracle(toks, cfg, sd), dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_each_mixer_and_feed_forward_alone(device, dtype):
+    """Single-layer models: each mixer without a feed-forward, each
+    feed-forward kind, the token input on and off."""
+    _one_layer(device, dtype, par(), None)
+    _one_layer(device, dtype, delta(3, 8), None)
+    _one_layer(device, dtype, delta(), dense(), side=5)
+    _one_layer(device, dtype, delta(), moe(), side=0)
+    _one_layer(device, dtype, par(size=0, pool=0, rot=0), moe(top=3), side=4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_state_space_mechanism(device):
+    """Convolution tail, softplus step, scalar decay, skip term and the gate
+    before the grouped norm, against the oracle's token loop."""
+    torch.manual_seed(9)
+    m = par(sh=4, svd=6, state=5, groups=2, ng=2, conv=4)["right"]
+    W, T, eps = 20, 15, 1e-5
+    cfg = make_cfg([(par(sh=4, svd=6, state=5, groups=2, ng=2, conv=4),
+                     None)], width=W, side=0)
+    sd = make_weights(cfg, 4)
+    w = O.layer_weights(sd, 0)
+    u = torch.randn(T, W).to(torch.bfloat16)
+    want = O.ssd(u.to(F64), w, m, eps, "mix.right.")
+    mc = ModelConfig.from_hf(cfg)
+    mc.compute_dtype = "float32"
+    mc.rms_eps = eps
+    ex = RingExecutor(mc, 0, 1, device, mb_size=2, smax=32,
+                      init_weights=False, use_graphs=False)
+    ex.model.load_state_dict(sd)
+    kv, lw = ex.kvs[0], ex.model.layers[0]
+    outs = []
+    for p0, n in ((0, 6), (6, 1), (7, 2), (9, 6)):     # portions carry state
+        pos = torch.tensor([p0], dtype=torch.int32, device=device)
+        slot = torch.tensor([1], dtype=torch.int32, device=device)
+        ln = torch.tensor([n], dtype=torch.int32, device=device)
+        outs.append(ex.model._ssd(u[p0:p0 + n].float().to(device), lw, m, kv,
+                                  0, pos, n, ln, slot))
+    close(torch.cat(outs), want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_delta_rule_mechanism(device):
+    """Both state terms read the old state; the unit key, the decay through
+    the low-rank path and the removal rate, against the oracle's loop."""
+    torch.manual_seed(10)
+    m = delta(3, 6)
+    W, T, eps = 18, 14, 1e-5
+    cfg = make_cfg([(m, None)], width=W, side=0)
+    sd = make_weights(cfg, 5)
+    u = torch.randn(T, W).to(torch.bfloat16)
+    want = O.general_delta(u.to(F64), O.layer_weights(sd, 0), m, eps)
+    ex = executor(cfg, sd, device, "float32", slots=2, smax=32)
+    kv, lw = ex.kvs[0], ex.model.layers[0]
+    outs = []
+    for p0, n in ((0, 5), (5, 1), (6, 1), (7, 7)):
+        pos = torch.tensor([p0], dtype=torch.int32, device=device)
+        slot = torch.tensor([0], dtype=torch.int32, device=device)
+        ln = torch.tensor([n], dtype=torch.int32, device=device)
+        outs.append(ex.model._delta(u[p0:p0 + n].float().to(device), lw, m,
+                                    kv, 0, pos, n, ln, slot))
+    close(torch.cat(outs), want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("rows", [5, 90])
+def test_expert_routing_mechanism(device, rows):
+    """Top-k by logit with the bias, softmax over the chosen logits only,
+    clamped gate/up with separate limits for routed and shared experts;
+    few rows (grouped path) and many (per-expert path)."""
+    torch.manual_seed(11)
+    ff = moe(experts=6, top=3, ff=16, limit=0.7, shared=8, slimit=0.4)
+    W = 24
+    cfg = make_cfg([(delta(), ff)], width=W, side=0)
+    sd = make_weights(cfg, 6)
+    u = (torch.randn(rows, W) * 2).to(torch.bfloat16)
+    want = O.moe_ff(u.to(F64), O.layer_weights(sd, 0), ff)
+    for dtype in ("float32", "bfloat16"):
+        ex = executor(cfg, sd, device, dtype, slots=1, smax=16)
+        x = u.to(device) if dtype == "bfloat16" else u.float().to(device)
+        close(ex.model._moe(x, ex.model.layers[0], ff), want, dtype)
+
+
+# ---------- whole model ----------
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_logits_and_first_tokens(device, dtype):
+    cfg = make_cfg(BASE)
+    sd = make_weights(cfg, 1, dtype=dtype)
+    ex = executor(cfg, sd, device, dtype)
+    toks = tokens(50, 83, 1)
+    want = oracle(toks, cfg, sd)
+    got = ex.prefill_slots([2], [toks], want=[list(range(50))])[0]
+    close(got, want, dtype)
+    one = ex.prefill_slots([0], [toks[:1]], want=[[0]])[0]
+    close(one, want[:1], dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_residual_after_every_layer(device):
+    cfg = make_cfg(BASE)
+    sd = make_weights(cfg, 2)
+    toks = tokens(17, 83, 2)
+    res = []
+    O.forward(toks.tolist(), cfg, sd, res)
+    for n in range(1, 5):
+        ex = executor(cfg, sd, device)
+        h = ex.model.embed_tokens(toks.view(1, -1).to(device)).clone()
+        ex.model.prefill_window(h, list(range(n)), ex.kvs[0], 0)
+        close(h[0], res[n - 1])
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_prefill_vs_token_by_token_and_long_decode(device):
+    """A one-token prompt followed by decoding every other token equals the
+    prompt taken whole; decoding runs far past every window and block."""
+    cfg = make_cfg(BASE)
+    sd = make_weights(cfg, 3)
+    toks = tokens(70, 83, 3)
+    want = oracle(toks, cfg, sd)
+    ex = executor(cfg, sd, device)
+    got = [ex.prefill_slots([1], [toks[:1]], want=[[0]])[0][0].float().cpu()]
+    for t in range(1, 70):
+        got.append(decode_steps(ex, {1: toks[t]})[1])
+    close(torch.stack(got), want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("chunk", [2, 3, 7, 32])
+def test_portions(device, chunk):
+    """The prompt cut into portions (the executor's position chunks and
+    continued prefill calls) gives the logits of the whole prompt."""
+    cfg = make_cfg(BASE)
+    sd = make_weights(cfg, 4)
+    toks = tokens(45, 83, 4)
+    want = oracle(toks, cfg, sd)
+    ex = executor(cfg, sd, device)
+    got = ex.prefill_slots([3], [toks], want=[list(range(45))],
+                           chunk=chunk)[0]
+    close(got, want)
+    ex2 = executor(cfg, sd, device)
+    parts, at = [], 0
+    while at < 45:
+        n = min(chunk + at % 3, 45 - at)
+        parts.append(ex2.prefill_slots([0], [toks[at:at + n]],
+                                       want=[list(range(n))],
+                                       start=[at])[0])
+        at += n
+    close(torch.cat(parts), want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_unequal_batch_equals_each_alone(device, dtype):
+    cfg = make_cfg(BASE)
+    sd = make_weights(cfg, 5, dtype=dtype)
+    ps = [tokens(n, 83, 10 + n) for n in (33, 2, 19, 1)]
+    wants = [oracle(p, cfg, sd) for p in ps]
+    ex = executor(cfg, sd, device, dtype, slots=5)
+    slots = [4, 0, 2, 3]
+    keep = [n - 6 if n > 8 else n for n in (33, 2, 19, 1)]
+    got = ex.prefill_slots(slots, [p[:k] for p, k in zip(ps, keep)],
+                           want=[list(range(k)) for k in keep], chunk=8)
+    for g, w, k in zip(got, wants, keep):
+        close(g, w[:k], dtype)
+    # the two long requests decode on together; the short ones have ended
+    for i in range(6):
+        lg = decode_steps(ex, {4: ps[0][27 + i], 2: ps[2][13 + i]})
+        close(lg[4:5], wants[0][27 + i].view(1, -1), dtype)
+        close(lg[2:3], wants[2][13 + i].view(1, -1), dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_slot_freed_and_used_again(device):
+    """A slot that held a long request is reused by a short one without any
+    reset: stale keys, pooled entries, convolution tails and recurrent
+    states of the old request must not reach the new one."""
+    cfg = make_cfg(BASE)
+    sd = make_weights(cfg, 6)
+    ex = executor(cfg, sd, device, slots=2)
+    a, b = tokens(60, 83, 21), tokens(25, 83, 22)
+    ex.prefill_slots([1], [a[:55]], want=[[54]])
+    for t in range(55, 60):
+        decode_steps(ex, {1: a[t]})
+    wb = oracle(b, cfg, sd)
+    ex.kvs[0].pos[1] = 0
+    got = ex.prefill_slots([1], [b[:20]], want=[list(range(20))])[0]
+    close(got, wb[:20])
+    for t in range(20, 25):
+        close(decode_steps(ex, {1: b[t]})[1:2], wb[t].view(1, -1))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_other_sizes(device, dtype):
+    """Sizes and constants in other relations: as many key heads as query
+    heads and a single one, one group / several, one norm group / several,
+    rotation of a part of the head and none, pool 1, window without pool and
+    no window, two taps and one, top-1 routing, no shared expert, layers
+    without a feed-forward, no token input, odd widths."""
+    cases = [
+        ([(par(heads=3, kv=3, dim=10, vdim=14, size=5, pool=1, rot=4,
+               sh=2, svd=10, state=12, groups=2, ng=1, conv=2), None),
+          (delta(1, 12), moe(experts=3, top=1, ff=8, shared=0))], 36, 0),
+        ([(delta(4, 4), dense(20)),
+          (par(heads=4, kv=1, dim=8, vdim=8, size=11, pool=0, rot=8,
+               sh=6, svd=4, state=3, groups=3, ng=3, conv=1), dense(9))],
+         30, 7),
+        ([(par(heads=2, kv=1, dim=12, vdim=4, size=0, pool=0, rot=0,
+               sh=1, svd=16, state=40, groups=1, ng=4, conv=5),
+           moe(experts=7, top=7, ff=8, limit=0.5, shared=16, slimit=2.0))],
+         28, 3),
+    ]
+    for layers, width, side in cases:
+        cfg = make_cfg(layers, width=width, vocab=61, side=side, eps=1e-6)
+        sd = make_weights(cfg, width, dtype=dtype)
+        ex = executor(cfg, sd, device, dtype, slots=3, smax=96)
+        a, b = tokens(40, 61, 1), tokens(9, 61, 2)
+        wa, wb = oracle(a, cfg, sd), oracle(b, cfg, sd)
+        got = ex.prefill_slots([2, 0], [a[:34], b[:7]],
+                               want=[list(range(34)), [0, 6]], chunk=16)
+        close(got[0], wa[:34], dtype)
+        close(got[1], wb[[0, 6]], dtype)
+        for i in range(2):
+            lg = decode_steps(ex, {2: a[34 + i], 0: b[7 + i]})
+            close(lg[2:3], wa[34 + i].view(1, -1), dtype)
+            close(lg[0:1], wb[7 + i].view(1, -1), dtype)
+        for i in range(2, 6):      # the short request has ended
+            lg = decode_steps(ex, {2: a[34 + i]})
+            close(lg[2:3], wa[34 + i].view(1, -1), dtype)
+
+
+@pytest.mark.gpu
+def test_decode_graph_replays_match_eager():
+    """Captured decode steps, replayed with eager prefills and host syncs in
+    between, equal the eager steps every time (warm-up runs of the capture
+    must not advance any slot's state)."""
+    cfg = make_cfg(BASE)
+    sd = make_weights(cfg, 7, dtype="bfloat16")
+    a, b = tokens(40, 83, 31), tokens(30, 83, 32)
+    runs = []
+    for graphs in (False, True):
+        mc = ModelConfig.from_hf(cfg)
+        mc.compute_dtype = "bfloat16"
+        ex = RingExecutor(mc, 0, 1, "cuda:0", mb_size=3, smax=128,
+                          init_weights=False, use_graphs=graphs)
+        ex.model.load_state_dict(sd)
+        out = [ex.prefill_slots([1], [a[:30]], want=[[0, 29]])[0].float().cpu()]
+        for t in range(30, 35):
+            out.append(decode_steps(ex, {1: a[t]})[1:2])
+        out.append(ex.prefill_slots([2], [b[:25]],
+                                    want=[[3, 24]])[0].float().cpu())
+        for t in range(5):
+            lg = decode_steps(ex, {1: a[35 + t], 2: b[25 + t]})
+            out.append(lg[1:3])
+            torch.cuda.synchronize()
+        runs.append(torch.cat(out))
+    torch.testing.assert_close(runs[1], runs[0], atol=2e-2, rtol=2e-2)
+    want = oracle(a, cfg, sd)
+    close(runs[1][2:3], want[30].view(1, -1), "bfloat16")
+
+
+# ---------- generation through the scheduler, trace replay ----------
+
+def write_checkpoint(path: Path, cfg, sd):
+    from safetensors.torch import save_file
+    path.mkdir(parents=True, exist_ok=True)
+    (path / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in sd.items()},
+              str(path / "model.safetensors"))
+
+
+def oracle_greedy(prompt, n, cfg, sd):
+    seq = list(prompt)
+    for _ in range(n):
+        seq.append(int(O.forward(seq, cfg, sd)[-1].argmax()))
+    return seq[len(prompt):]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_slot_scheduler(tmp_path, device,
+                                                  monkeypatch):
+    """Requests queued at the shard runtime are admitted into slots (more
+    requests than slots), prefilled, decoded as one batch with idle rows in
+    it and sampled greedily; every token equals the oracle's argmax."""
+    if device == "cpu":
+        monkeypatch.setattr(torch.cuda, "is_available", lambda: False)
+    from dnet_amd.core.types import ShardLoadModelRequest
+    from dnet_amd.shard.runtime import ShardRuntime
+    cfg = make_cfg(BASE[:3], vocab=59)
+    sd = make_weights(cfg, 15)
+    write_checkpoint(tmp_path / "m", cfg, sd)
+    emitted: dict = {}
+
+    class Cap:
+        def send(self, frame):
+            emitted.setdefault(frame["nonce"], []).append(
+                (frame["token_id"], frame["finished"]))
+
+        def close(self):
+            pass
+
+    rt = ShardRuntime("probe")
+    monkeypatch.setattr(rt.settings.storage, "repack_on_load", False)
+    rt._load(ShardLoadModelRequest(
+        model_path=str(tmp_path / "m"), total_layers=3, layers=[0, 1, 2],
+        max_batch=2, max_seq=96, dtype="float32"))
+    assert (rt.executor.device.type == "cuda") == device.startswith("cuda")
+    rt._callback = Cap()
+    prompts = {"a": tokens(9, 59, 1), "b": tokens(2, 59, 2),
+               "c": tokens(23, 59, 3)}
+    n_new = {"a": 6, "b": 9, "c": 4}
+    for name in ("a", "b", "c"):            # c waits for a slot to free up
+        rt.infer_q.put({"nonce": name, "prompt_len": len(prompts[name]),
+                        "tokens": prompts[name].to(torch.int32).numpy()
+                        .tobytes(), "max_tokens": n_new[name],
+                        "stop_ids": [], "params": {}})
+    for _ in range(60):
+        rt._slots_tick()
+        if all(emitted.get(k) and emitted[k][-1][1] for k in prompts):
+            break
+    for name, p in prompts.items():
+        got = [t for t, _ in emitted[name]]
+        assert got == oracle_greedy(p.tolist(), n_new[name], cfg, sd), name
+    rt._unload()
+
+
+@pytest.mark.gpu
+def test_trace_replay_cli_gpu(tmp_path):
+    test_trace_replay_cli(tmp_path, "bfloat16")
+    test_trace_replay_cli(tmp_path / "f", "float32")
+
+
+def test_trace_replay_cli(tmp_path, dtype="float32"):
+    """bin/trace_run on a tiny checkpoint: a prompt batch of unequal
+    requests (more than the initial slot count), decode steps together, a
+    request that sits steps out, requests that end early, a slot used
+    again by a new request."""
+    cfg = make_cfg(BASE[:3], vocab=53)
+    sd = make_weights(cfg, 16, dtype=dtype)
+    write_checkpoint(tmp_path / "m", cfg, sd)
+    a, b = tokens(14, 53, 1).tolist(), tokens(4, 53, 2).tolist()
+    c, d = tokens(12, 53, 3).tolist(), tokens(6, 53, 4).tolist()
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:11], "want": [0, 10]},
+                                {"id": "b", "tokens": b[:2], "want": []},
+                                {"id": "c", "tokens": c[:10], "want": [9]}],
+         "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[11:12], "want": [0]},
+                                {"id": "b", "tokens": b[2:3], "want": [0]}],
+         "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[12:13], "want": []},
+                                {"id": "b", "tokens": b[3:4], "want": [0]}],
+         "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[13:14], "want": [0]}],
+         "end": ["a"]},
+        {"step": 4, "entries": [{"id": "c", "tokens": c[10:11], "want": [0]}],
+         "end": []},
+        {"step": 5, "entries": [{"id": "d", "tokens": d[:5], "want": [4]}],
+         "end": []},
+        {"step": 6, "entries": [{"id": "c", "tokens": c[11:12], "want": [0]},
+                                {"id": "d", "tokens": d[5:6], "want": [0]}],
+         "end": ["c", "d"]},
+    ]
+    root = Path(__file__).resolve().parents[1]
+    r = subprocess.run(
+        [sys.executable, str(root / "bin" / "trace_run"), "--model",
+         str(tmp_path / "m"), "--dtype", dtype, "--out",
+         str(tmp_path / "out"), "--max-tokens", "48", "--max-batch", "2"],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+        capture_output=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [
+        f"done {i}" for i in range(7)]
+    w = {n: O.forward(t, cfg, sd) for n, t in
+         (("a", a), ("b", b), ("c", c), ("d", d))}
+    import numpy as np
+
+    def rd(i):
+        return torch.from_numpy(np.fromfile(tmp_path / "out" / f"{i}.f32",
+                                            dtype="<f4").reshape(-1, 53))
+    close(rd(0), torch.cat([w["a"][[0, 10]], w["c"][9:10]]), dtype)
+    close(rd(1), torch.stack([w["a"][11], w["b"][2]]), dtype)
+    close(rd(2), w["b"][3:4], dtype)
+    close(rd(3), w["a"][13:14], dtype)
+    close(rd(4), w["c"][10:11], dtype)
+    close(rd(5), w["d"][4:5], dtype)
+    close(rd(6), torch.stack([w["c"][11], w["d"][5]]), dtype)
+
+
+def test_pipeline_stages_are_refused():
+    """Every layer reads the token ids; the ring hops carry the residual
+    only, so a second stage is refused at construction."""
+    mc = ModelConfig.from_hf(make_cfg(BASE))
+    from dnet_amd.parallel.ring import RingPlan
+    with pytest.raises(NotImplementedError):
+        RingExecutor(mc, 0, 2, "cpu", plan=RingPlan.contiguous(4, 2),
+                     init_weights=False, use_graphs=False)
+
+
+def test_synthetic_preset_runs():
+    """The benchmark preset builds with seeded random weights and generates
+    the same tokens whatever the slot a prompt sits in."""
+    from dnet_amd.models import PRESETS
+    mc = ModelConfig.from_hf(dict(PRESETS["gegorax-tiny"]))
+    ex = RingExecutor(mc, 0, 1, "cpu", mb_size=2, smax=96, seed=3,
+                      use_graphs=False)
+    toks = torch.randint(0, 256, (1, 2, 30),
+                         generator=torch.Generator().manual_seed(1))
+    toks[0, 1] = toks[0, 0]
+    first = ex.prefill(toks)
+    gen = ex.decode_rounds(6)
+    assert torch.equal(first[0, 0], first[0, 1])
+    assert torch.equal(gen[0, 0], gen[0, 1])
