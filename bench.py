@@ -53,11 +53,42 @@ _COMPARE_SIZES = [("2k", 2048, 16, 4, 128, 8192),
                   ("5k", 5120, 64, 8, 128, 25600)]
 
 
-def compare_posudra(args, device):
-    """Prefill and decode throughput of posudra beside the closest existing
-    family (qwen3: dense, grouped heads, q/k norm) at equal layer sizes,
-    bf16, random weights. One JSON line; the default workload is untouched."""
-    from dnet_amd.models.config import posudra_config
+def _family_hf(fam, W, H, KV, D, FF, layers, vocab, args):
+    """config.json-style description of ``fam`` at the given layer sizes."""
+    from dnet_amd.models.config import gegorax_config, posudra_config
+    if fam == "posudra":
+        return posudra_config(W, layers, H, KV, D, D, FF, vocab)
+    if fam == "gegorax":
+        # attention + state-space layers alternate with delta-rule layers;
+        # window half the prompt, 16-position pooled blocks; state-space and
+        # delta-rule heads of 64 channels over the model width; a per-layer
+        # token input of 256 channels; dense feed-forwards unless
+        # --compare-experts asks for a mixture in every second layer
+        E = args.compare_experts
+        return gegorax_config(
+            W, layers, vocab, H, KV, D, D, window=max(64, args.prompt_len // 2),
+            pool=16, ssm_heads=W // 64, ssm_vdim=64, ssm_state=128,
+            delta_heads=W // 64, delta_dim=64, ff=FF, experts=E,
+            top=min(4, E), expert_ff=FF // 8, shared_ff=FF // 8 if E else 0,
+            side_dim=256)
+    return dict(model_type="qwen3", hidden_size=W,
+                num_hidden_layers=layers, num_attention_heads=H,
+                num_key_value_heads=KV, head_dim=D,
+                intermediate_size=FF, vocab_size=vocab,
+                rope_theta=1000000.0, rms_norm_eps=1e-6)
+
+
+# family -> the closest existing family it is measured beside
+_COMPARE_WITH = {"posudra": "qwen3", "gegorax": "posudra"}
+
+
+def compare_family(args, device):
+    """Prefill and decode throughput of a family beside the closest existing
+    one (posudra: qwen3 — dense, grouped heads, q/k norm; gegorax: posudra —
+    one norm feeding parallel branches, fp32 residual, per-layer sizes) at
+    equal layer sizes, bf16, random weights. One JSON line; the default
+    workload is untouched."""
+    new, old = args.compare_family, _COMPARE_WITH[args.compare_family]
     layers, vocab = args.compare_layers, 32768
     B, T, Bd = args.compare_prefill_batch, args.prompt_len, args.mb_size
     rows = []
@@ -66,15 +97,8 @@ def compare_posudra(args, device):
             continue
         row = {"size": name, "width": W, "heads": H, "kv_heads": KV,
                "head_dim": D, "ff": FF, "layers": layers}
-        for fam in ("posudra", "qwen3"):
-            if fam == "posudra":
-                hf = posudra_config(W, layers, H, KV, D, D, FF, vocab)
-            else:
-                hf = dict(model_type="qwen3", hidden_size=W,
-                          num_hidden_layers=layers, num_attention_heads=H,
-                          num_key_value_heads=KV, head_dim=D,
-                          intermediate_size=FF, vocab_size=vocab,
-                          rope_theta=1000000.0, rms_norm_eps=1e-6)
+        for fam in (new, old):
+            hf = _family_hf(fam, W, H, KV, D, FF, layers, vocab, args)
             cfg = ModelConfig.from_hf(hf)
             g = torch.Generator().manual_seed(7)
             # prefill: B prompts of T tokens, eager (as serving runs it)
@@ -110,7 +134,7 @@ def compare_posudra(args, device):
             torch.cuda.empty_cache()
         rows.append(row)
     print(json.dumps({
-        "metric": "posudra vs qwen3 at equal layer sizes: prefill and "
+        "metric": f"{new} vs {old} at equal layer sizes: prefill and "
                   "decode tokens/s (1 GPU, bf16)",
         "dtype": "bf16", "data": "synthetic (random tokens, random-init "
                                  "weights)",
@@ -149,11 +173,15 @@ def main():
     ap.add_argument("--residency", type=int, default=0,
                     help="GPU-resident layers per rank (0=all; <local layers "
                          "enables host-DRAM weight streaming)")
-    ap.add_argument("--compare-family", default="", choices=["", "posudra"],
+    ap.add_argument("--compare-family", default="",
+                    choices=["", "posudra", "gegorax"],
                     help="instead of the default workload: throughput of "
                          "this family beside its closest existing one at "
                          "equal layer sizes")
     ap.add_argument("--compare-layers", type=int, default=8)
+    ap.add_argument("--compare-experts", type=int, default=0,
+                    help="gegorax: experts of the mixture feed-forward in "
+                         "every second layer (0 = dense feed-forwards)")
     ap.add_argument("--compare-prefill-batch", type=int, default=8)
     ap.add_argument("--compare-sizes", default="",
                     help="comma list out of 2k,4k,5k (default: all)")
@@ -169,7 +197,7 @@ def main():
                         + args.warmup + 64)
         if args.mb_size == 64:
             args.mb_size = 32
-        compare_posudra(args, device)
+        compare_family(args, device)
         return
 
     quant = None

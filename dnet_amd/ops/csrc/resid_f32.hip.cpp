@@ -151,6 +151,8 @@ __global__ __launch_bounds__(256) void xielu_kernel(
   }
 }
 
+constexpr int kMaxRot = 128;   // rotated pairs per head (head size <= 256)
+
 // qkv row layout: [q: nq*d | k: nkv*d | v: nkv*dv]. Token (b,t) = row b*T+t
 // sits at position pos[b]+t of cache row slots[b] (default b); tokens with
 // t >= lens[b] are padding: q is still written, the cache is not touched.
@@ -213,9 +215,51 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
     // one wave per head; weights are per head-dim element
     const int wid = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
     const int nw = blockDim.x / kWave;
+    // every head of the row turns by the same angles: one sincos per pair
+    __shared__ float rot_c[kMaxRot], rot_s[kMaxRot];
+    for (int i = threadIdx.x; i < nrot; i += blockDim.x)
+      sincosf((float)p * rot_freq[i], &rot_s[i], &rot_c[i]);
+    if (nrot > 0) __syncthreads();
     for (int hh = wid; hh < nq + nkv; hh += nw) {
       const bool isq = hh < nq;
       const T* hs = isq ? src + hh * d : src + NQ + (hh - nq) * d;
+      if (!isq && !keep) continue;            // wave-uniform
+      const float* wv = isq ? qw : kw;
+      T* dst = isq ? qo + hh * d
+                   : kc + kbase + (int64_t)(hh - nq) * Smax * d;
+      if (d <= 4 * kWave) {
+        // one read: a lane keeps channel pairs (2i, 2i+1), i = lane, lane+64
+        float v0[2], v1[2];
+        float ss = 0.f;
+#pragma unroll
+        for (int qd = 0; qd < 2; ++qd) {
+          const int e0 = 2 * (lane + kWave * qd);
+          v0[qd] = e0 < d ? ldf<T>(hs + e0) : 0.f;
+          v1[qd] = e0 + 1 < d ? ldf<T>(hs + e0 + 1) : 0.f;
+          ss += v0[qd] * v0[qd] + v1[qd] * v1[qd];
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        const float r = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+        for (int qd = 0; qd < 2; ++qd) {
+          const int pr = lane + kWave * qd;
+          const int e0 = 2 * pr, e1 = e0 + 1;
+          if (e0 >= d) continue;
+          float a0 = v0[qd] * r * wv[e0];
+          float a1 = e1 < d ? v1[qd] * r * wv[e1] : 0.f;
+          if (pr < nrot && e1 < d) {
+            // pairs i < nrot turn by position * rot_freq[i], in fp32
+            const float sn = rot_s[pr], cs = rot_c[pr];
+            const float u0 = a0 * cs - a1 * sn;
+            a1 = a1 * cs + a0 * sn;
+            a0 = u0;
+          }
+          stf<T>(dst + e0, a0);
+          if (e1 < d) stf<T>(dst + e1, a1);
+        }
+        continue;
+      }
       float ss = 0.f;
       for (int e = lane; e < d; e += kWave) {
         const float v = ldf<T>(hs + e);
@@ -224,30 +268,18 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
       const float r = 1.0f / sqrtf(ss / (float)d + eps);
-      const float* wv = isq ? qw : kw;
-      T* dst = isq ? qo + hh * d
-                   : kc + kbase + (int64_t)(hh - nq) * Smax * d;
-      if (!isq && !keep) continue;
-      if (nrot > 0) {
-        // lanes own channel pairs (2i, 2i+1); pairs i < nrot turn by the
-        // angle position * rot_freq[i], computed and applied in fp32
-        for (int pr = lane; 2 * pr < d; pr += kWave) {
-          const int e0 = 2 * pr, e1 = e0 + 1;
-          float v0 = ldf<T>(hs + e0) * r * wv[e0];
-          float v1 = e1 < d ? ldf<T>(hs + e1) * r * wv[e1] : 0.f;
-          if (pr < nrot && e1 < d) {
-            float sn, cs;
-            sincosf((float)p * rot_freq[pr], &sn, &cs);
-            const float u0 = v0 * cs - v1 * sn;
-            v1 = v1 * cs + v0 * sn;
-            v0 = u0;
-          }
-          stf<T>(dst + e0, v0);
-          if (e1 < d) stf<T>(dst + e1, v1);
+      for (int pr = lane; 2 * pr < d; pr += kWave) {
+        const int e0 = 2 * pr, e1 = e0 + 1;
+        float a0 = ldf<T>(hs + e0) * r * wv[e0];
+        float a1 = e1 < d ? ldf<T>(hs + e1) * r * wv[e1] : 0.f;
+        if (pr < nrot && e1 < d) {
+          const float sn = rot_s[pr], cs = rot_c[pr];
+          const float u0 = a0 * cs - a1 * sn;
+          a1 = a1 * cs + a0 * sn;
+          a0 = u0;
         }
-      } else {
-        for (int e = lane; e < d; e += kWave)
-          stf<T>(dst + e, ldf<T>(hs + e) * r * wv[e]);
+        stf<T>(dst + e0, a0);
+        if (e1 < d) stf<T>(dst + e1, a1);
       }
     }
   }
@@ -384,24 +416,27 @@ __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(
   }
 }
 
-// kind 0: max(z, 0)^2, kind 1: tanh(z); columns [col0, col0+n) of x (stride ld)
-template <typename T>
+// kind 0: max(z, 0)^2, kind 1: tanh(z); columns [col0, col0+n) of x (stride
+// ld); W = 4 when ld, col0 and n are multiples of 4
+template <typename T, int W>
 __global__ __launch_bounds__(256) void act_slice_kernel(
     const T* __restrict__ x, const int64_t ld, const int col0,
     T* __restrict__ y, const int n, const int64_t total, const int kind) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * blockDim.x) {
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * W;
+       i < total; i += (int64_t)gridDim.x * blockDim.x * W) {
     const int64_t row = i / n;
     const int c = (int)(i % n);
-    const float z = ldf<T>(x + row * ld + col0 + c);
-    float v;
-    if (kind == 0) {
-      const float t = fmaxf(z, 0.f);
-      v = t * t;
-    } else {
-      v = tanhf(z);
+    vecf<W> v = ldw<W, T>(x + row * ld + col0 + c);
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      if (kind == 0) {
+        const float t = fmaxf(v.v[j], 0.f);
+        v.v[j] = t * t;
+      } else {
+        v.v[j] = tanhf(v.v[j]);
+      }
     }
-    stf<T>(y + i, v);
+    stw<W, T>(y + i, v);
   }
 }
 
@@ -556,7 +591,8 @@ void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
   if (rot_freq.has_value()) {
     DNET_CHECK(per_head, "rotation comes with the per-head norm");
     DNET_CHECK(is_f32(*rot_freq) && rot_freq->is_contiguous() &&
-                   rot_freq->numel() * 2 <= d, "rot_freq fp32 [<= d/2]");
+                   rot_freq->numel() * 2 <= d &&
+                   rot_freq->numel() <= kMaxRot, "rot_freq fp32 [<= d/2]");
     nrot = (int)rot_freq->numel();
   }
   DNET_CHECK(T > 0 && M % T == 0, "rows = B*T");
@@ -696,17 +732,16 @@ void act_slice(torch::Tensor x, int64_t col0, torch::Tensor y, int64_t kind) {
   const int64_t total = y.numel();
   if (total == 0) return;
   auto st = current_stream();
-  if (is_bf16(x))
-    hipLaunchKernelGGL((act_slice_kernel<short>), dim3(ew_blocks(total)),
-                       dim3(256), 0, st, (const short*)x.data_ptr(),
-                       x.size(1), (int)col0, (short*)y.data_ptr(), n, total,
-                       (int)kind);
-  else if (is_f32(x))
-    hipLaunchKernelGGL((act_slice_kernel<float>), dim3(ew_blocks(total)),
-                       dim3(256), 0, st, (const float*)x.data_ptr(),
-                       x.size(1), (int)col0, (float*)y.data_ptr(), n, total,
-                       (int)kind);
+  const bool v4 = x.size(1) % 4 == 0 && col0 % 4 == 0 && n % 4 == 0;
+  const int blocks = ew_blocks(v4 ? total / 4 : total);
+#define AS(TT, WW)                                                           \
+  hipLaunchKernelGGL((act_slice_kernel<TT, WW>), dim3(blocks), dim3(256), 0, \
+                     st, (const TT*)x.data_ptr(), x.size(1), (int)col0,      \
+                     (TT*)y.data_ptr(), n, total, (int)kind)
+  if (is_bf16(x)) { if (v4) AS(short, 4); else AS(short, 1); }
+  else if (is_f32(x)) { if (v4) AS(float, 4); else AS(float, 1); }
   else DNET_CHECK(false, "act_slice: dtype");
+#undef AS
 }
 
 void gelu_gather_mul(torch::Tensor z, torch::Tensor table,

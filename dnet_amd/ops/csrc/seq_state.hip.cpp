@@ -18,7 +18,7 @@
 // The two scans share one layout: a workgroup owns one head (or a slice of
 // its value columns) of one batch row and walks the tokens in order. The
 // state matrix [rows x columns] is spread as: thread (column j, slice s)
-// keeps rows [32 s, 32 s + 32) of column j in registers; the slices of a
+// keeps rows [R s, R s + R) of column j in registers (R = 32, 16 or 8); the slices of a
 // column are neighbouring lanes, so the two per-token reductions over rows
 // are in-register sums plus a few lane shuffles. Per-token vectors (B, C /
 // r, k, w, ...) are staged through LDS in chunks of tokens, with all their
@@ -36,7 +36,13 @@ template <typename T> __device__ __forceinline__ void sts(T* p, float v);
 template <> __device__ __forceinline__ void sts<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void sts<short>(short* p, float v) { *p = f2bits(v); }
 
-constexpr int kRows = 32;      // state rows per thread
+// State rows per thread R is 32, 16 or 8 (fewer rows = more lanes per column =
+// more waves in flight when batch x heads is small). LDS pitch of one R-row
+// slice: 4 spare floats shift neighbouring slices by four banks, so the 16 B
+// reads of the slices of a column never collide.
+template <int R> __host__ __device__ inline int padded(int r) {
+  return (r / R) * (R + 4) + (r % R);
+}
 
 struct Geo {
   const int* pos;
@@ -90,35 +96,145 @@ __global__ __launch_bounds__(128) void kv_pool_kernel(
 }
 
 // ---- causal convolution ----------------------------------------------------
-// grid (channel tiles, B*T). state [Bc, taps-1, C]: entry j of a slot holds
-// the input at position pos - (taps-1) + j (positions < 0 count as zero).
-template <typename T>
+// grid (channel tiles, B*T), CW channels per thread (4 when the row stride,
+// the first column and C are multiples of 4: 8 B / 16 B accesses). state
+// [Bc, taps-1, C]: entry j of a slot holds the input at position
+// pos - (taps-1) + j (positions < 0 count as zero).
+template <typename T, int CW>
 __global__ __launch_bounds__(256) void conv_silu_kernel(
     const T* __restrict__ x, const int64_t ld, const int col0,
     const float* __restrict__ w, const float* __restrict__ bias,
     const T* __restrict__ state, float* __restrict__ y, const Geo g,
     const int C, const int taps) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * CW;
   if (c >= C) return;
   const int64_t row = blockIdx.y;
   const int b = (int)(row / g.T), t = (int)(row % g.T);
   int p0, n, slot;
-  if (!row_geo(g, b, p0, n, slot) || t >= n) {
-    y[row * C + c] = 0.f;
-    return;
-  }
-  float acc = bias[c];
-  for (int j = 0; j < taps; ++j) {
-    const int tt = t - (taps - 1) + j;
-    float v = 0.f;
-    if (tt >= 0) {
-      v = lds<T>(x + ((int64_t)b * g.T + tt) * ld + col0 + c);
-    } else if (p0 + tt >= 0) {
-      v = lds<T>(state + ((int64_t)slot * (taps - 1) + (taps - 1 + tt)) * C + c);
+  float acc[CW];
+  const bool on = row_geo(g, b, p0, n, slot) && t < n;
+#pragma unroll
+  for (int e = 0; e < CW; ++e) acc[e] = on ? bias[c + e] : 0.f;
+  if (on) {
+    for (int j = 0; j < taps; ++j) {
+      const int tt = t - (taps - 1) + j;
+      const T* src = nullptr;
+      if (tt >= 0) {
+        src = x + ((int64_t)b * g.T + tt) * ld + col0 + c;
+      } else if (p0 + tt >= 0) {
+        src = state + ((int64_t)slot * (taps - 1) + (taps - 1 + tt)) * C + c;
+      }
+      if (src == nullptr) continue;
+      float v[CW];
+      if constexpr (CW == 4 && sizeof(T) == 2) {
+        const short4v q = *reinterpret_cast<const short4v*>(src);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = bits2f(q.x[e]);
+      } else if constexpr (CW == 4) {
+        const float4 q = *reinterpret_cast<const float4*>(src);
+        v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+      } else {
+        v[0] = lds<T>(src);
+      }
+#pragma unroll
+      for (int e = 0; e < CW; ++e)
+        acc[e] = fmaf(w[(c + e) * taps + j], v[e], acc[e]);
     }
-    acc = fmaf(w[c * taps + j], v, acc);
+#pragma unroll
+    for (int e = 0; e < CW; ++e) acc[e] = acc[e] * sigmoid_a(acc[e]);
   }
-  y[row * C + c] = acc * sigmoid_a(acc);
+  if constexpr (CW == 4) {
+    *reinterpret_cast<float4*>(y + row * C + c) =
+        make_float4(acc[0], acc[1], acc[2], acc[3]);
+  } else {
+    y[row * C + c] = acc[0];
+  }
+}
+
+// Token-tiled variant for taps <= 4: grid (channel tiles, B * token tiles).
+// A thread walks kConvTile consecutive tokens of its CW channels with the
+// taps and the sliding window of inputs in registers, so every input is read
+// once and the weights once per tile.
+constexpr int kConvTile = 16;
+
+template <typename T, int CW>
+__device__ __forceinline__ void conv_load(const T* src, float (&v)[CW]) {
+  if constexpr (CW == 4 && sizeof(T) == 2) {
+    const short4v q = *reinterpret_cast<const short4v*>(src);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = bits2f(q.x[e]);
+  } else if constexpr (CW == 4) {
+    const float4 q = *reinterpret_cast<const float4*>(src);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  } else {
+    v[0] = lds<T>(src);
+  }
+}
+
+template <typename T, int CW, int TAPS>
+__global__ __launch_bounds__(256) void conv_silu_tile_kernel(
+    const T* __restrict__ x, const int64_t ld, const int col0,
+    const float* __restrict__ w, const float* __restrict__ bias,
+    const T* __restrict__ state, float* __restrict__ y, const Geo g,
+    const int C) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * CW;
+  if (c >= C) return;
+  const int ntile = (g.T + kConvTile - 1) / kConvTile;
+  const int b = blockIdx.y / ntile;
+  const int t0 = (blockIdx.y % ntile) * kConvTile;
+  const int t1 = min(t0 + kConvTile, g.T);
+  int p0, n, slot;
+  const bool valid = row_geo(g, b, p0, n, slot);
+  float wr[TAPS][CW], br[CW], win[TAPS][CW];
+#pragma unroll
+  for (int e = 0; e < CW; ++e) {
+    br[e] = bias[c + e];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) wr[j][e] = w[(c + e) * TAPS + j];
+  }
+  // inputs at t0-(TAPS-1) .. t0-1: earlier rows of this step, the slot's
+  // tail, or zero before position 0
+#pragma unroll
+  for (int j = 0; j < TAPS - 1; ++j) {
+    const int tt = t0 - (TAPS - 1) + j;
+#pragma unroll
+    for (int e = 0; e < CW; ++e) win[j][e] = 0.f;
+    if (!valid || t0 >= n) continue;
+    if (tt >= 0)
+      conv_load<T, CW>(x + ((int64_t)b * g.T + tt) * ld + col0 + c, win[j]);
+    else if (p0 + tt >= 0)
+      conv_load<T, CW>(
+          state + ((int64_t)slot * (TAPS - 1) + (TAPS - 1 + tt)) * C + c,
+          win[j]);
+  }
+#pragma unroll 4
+  for (int t = t0; t < t1; ++t) {
+    const int64_t row = (int64_t)b * g.T + t;
+    float acc[CW];
+    if (valid && t < n) {
+      conv_load<T, CW>(x + row * ld + col0 + c, win[TAPS - 1]);
+#pragma unroll
+      for (int e = 0; e < CW; ++e) {
+        float a = br[e];
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) a = fmaf(wr[j][e], win[j][e], a);
+        acc[e] = a * sigmoid_a(a);
+      }
+#pragma unroll
+      for (int j = 0; j < TAPS - 1; ++j)
+#pragma unroll
+        for (int e = 0; e < CW; ++e) win[j][e] = win[j + 1][e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < CW; ++e) acc[e] = 0.f;
+    }
+    if constexpr (CW == 4) {
+      *reinterpret_cast<float4*>(y + row * C + c) =
+          make_float4(acc[0], acc[1], acc[2], acc[3]);
+    } else {
+      y[row * C + c] = acc[0];
+    }
+  }
 }
 
 // grid (channel tiles, B): shift the slot's tail by its n new inputs
@@ -144,7 +260,7 @@ __global__ __launch_bounds__(256) void conv_state_kernel(
 // ---- state-space recurrence ------------------------------------------------
 // grid (heads * column tiles, B), block = JB columns x NS slices.
 // LDS per token of a chunk: B [NP], C [NP], x [JB], dt, decay.
-template <typename TD>
+template <typename TD, int R>
 __global__ __launch_bounds__(256) void ssd_scan_kernel(
     const float* __restrict__ xbc, const TD* __restrict__ dt_src,
     const int64_t dld, const int dcol0, const float* __restrict__ dt_bias,
@@ -160,7 +276,8 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(
   if (!row_geo(g, b, p0, n, slot)) return;
   const int grp = h / (heads / G);
   const int inner = heads * P, C = inner + 2 * G * N;
-  const int NP = NS * kRows;                    // padded state rows
+  const int NR = NS * R;                    // state rows incl. padding
+  const int NP = NS * (R + 4);                   // LDS pitch of one token
   const int jl = threadIdx.x / NS, sl = threadIdx.x % NS;
   const int j = j0 + jl;
   const bool col_ok = j < P;
@@ -172,11 +289,11 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(
   float* sDt = sX + TC * JB;                    // [TC]
   float* sDec = sDt + TC;                       // [TC]
 
-  float S[kRows];
+  float S[R];
   float* sp = state + (((int64_t)slot * heads + h) * N) * P;
 #pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int row = sl * kRows + r;
+  for (int r = 0; r < R; ++r) {
+    const int row = sl * R + r;
     S[r] = (p0 > 0 && col_ok && row < N) ? sp[(int64_t)row * P + j] : 0.f;
   }
   const float a_h = expf(a_log[h]), d_h = dskip[h], bias_h = dt_bias[h];
@@ -184,11 +301,11 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(
   for (int t0 = 0; t0 < n; t0 += TC) {
     const int tc = min(TC, n - t0);
     __syncthreads();                            // previous chunk consumed
-    for (int idx = threadIdx.x; idx < tc * NP; idx += blockDim.x) {
-      const int tt = idx / NP, r = idx % NP;
+    for (int idx = threadIdx.x; idx < tc * NR; idx += blockDim.x) {
+      const int tt = idx / NR, r = idx % NR;
       const float* src = xbc + ((int64_t)b * g.T + t0 + tt) * C + inner;
-      sB[idx] = r < N ? src[grp * N + r] : 0.f;
-      sC[idx] = r < N ? src[G * N + grp * N + r] : 0.f;
+      sB[tt * NP + padded<R>(r)] = r < N ? src[grp * N + r] : 0.f;
+      sC[tt * NP + padded<R>(r)] = r < N ? src[G * N + grp * N + r] : 0.f;
     }
     for (int idx = threadIdx.x; idx < tc * JB; idx += blockDim.x) {
       const int tt = idx / JB, c = idx % JB;
@@ -207,11 +324,11 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(
     for (int tt = 0; tt < tc; ++tt) {
       const float xj = sX[tt * JB + jl];
       const float dec = sDec[tt], dtx = sDt[tt] * xj;
-      const float4* bp = reinterpret_cast<const float4*>(sB + tt * NP + sl * kRows);
-      const float4* cp = reinterpret_cast<const float4*>(sC + tt * NP + sl * kRows);
+      const float4* bp = reinterpret_cast<const float4*>(sB + tt * NP + sl * (R + 4));
+      const float4* cp = reinterpret_cast<const float4*>(sC + tt * NP + sl * (R + 4));
       float acc = 0.f;
 #pragma unroll
-      for (int r4 = 0; r4 < kRows / 4; ++r4) {
+      for (int r4 = 0; r4 < R / 4; ++r4) {
         const float4 bv = bp[r4], cv = cp[r4];
         S[4 * r4 + 0] = fmaf(dec, S[4 * r4 + 0], dtx * bv.x);
         S[4 * r4 + 1] = fmaf(dec, S[4 * r4 + 1], dtx * bv.y);
@@ -231,8 +348,8 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(
   }
   if (col_ok) {
 #pragma unroll
-    for (int r = 0; r < kRows; ++r) {
-      const int row = sl * kRows + r;
+    for (int r = 0; r < R; ++r) {
+      const int row = sl * R + r;
       if (row < N) sp[(int64_t)row * P + j] = S[r];
     }
   }
@@ -240,8 +357,8 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(
 
 // ---- generalized delta rule ------------------------------------------------
 // grid (H * column tiles, B), block = JB value columns x NS key slices.
-// LDS per token of a chunk: r, k, w, au (= a*u), u [DP each], v [JB].
-template <typename T>
+// LDS per token of a chunk: r, k, w, a*k [DP each], v [JB], 1/(|k|^2+eps).
+template <typename T, int R>
 __global__ __launch_bounds__(256) void delta_scan_kernel(
     const T* __restrict__ src, const int64_t ld, const int r0, const int k0,
     const int v0, const int a0, const T* __restrict__ wl,
@@ -255,7 +372,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   const int b = blockIdx.y;
   int p0, n, slot;
   if (!row_geo(g, b, p0, n, slot)) return;
-  const int DP = NS * kRows;                    // padded key rows
+  const int DR = NS * R;                    // key rows incl. padding
+  const int DP = NS * (R + 4);                   // LDS pitch of one token
   const int jl = threadIdx.x / NS, sl = threadIdx.x % NS;
   const int j = j0 + jl;
   const bool col_ok = j < d;
@@ -266,15 +384,15 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   float* sR = sm;                               // [TC][DP]
   float* sK = sR + TC * DP;
   float* sW = sK + TC * DP;
-  float* sAU = sW + TC * DP;
-  float* sU = sAU + TC * DP;
-  float* sV = sU + TC * DP;                     // [TC][JB]
+  float* sAK = sW + TC * DP;                    // a * k
+  float* sV = sAK + TC * DP;                    // [TC][JB]
+  float* sRn = sV + TC * JB;                    // [TC] 1 / (sum k^2 + eps)
 
-  float S[kRows];
+  float S[R];
   float* sp = state + (((int64_t)slot * H + h) * d) * d;
 #pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int row = sl * kRows + r;
+  for (int r = 0; r < R; ++r) {
+    const int row = sl * R + r;
     S[r] = (p0 > 0 && col_ok && row < d) ? sp[(int64_t)row * d + j] : 0.f;
   }
   const int hd = h * d;
@@ -282,35 +400,25 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   for (int t0 = 0; t0 < n; t0 += TC) {
     const int tc = min(TC, n - t0);
     __syncthreads();                            // previous chunk consumed
-    // one wave per token: unit key needs the head's sum of squares
-    for (int tt = wid; tt < tc; tt += nw) {
+    // element-wise staging: every load of the chunk is in flight at once
+    for (int idx = threadIdx.x; idx < tc * DR; idx += blockDim.x) {
+      const int tt = idx / DR, i = idx % DR;
       const int64_t row = (int64_t)b * g.T + t0 + tt;
       const T* sr = src + row * ld;
-      float ss = 0.f;
-      for (int i = lane; i < d; i += kWave) {
-        const float kv = lds<T>(sr + k0 + hd + i);
-        ss += kv * kv;
+      float rv = 0.f, kv = 0.f, wv = 0.f, av = 0.f;
+      if (i < d) {
+        rv = lds<T>(sr + r0 + hd + i);
+        kv = lds<T>(sr + k0 + hd + i);
+        wv = expf(-decay_scale *
+                  sigmoid_a(lds<T>(wl + row * (int64_t)(H * d) + hd + i) +
+                            w0[hd + i]));
+        av = sigmoid_a(lds<T>(sr + a0 + hd + i) + ab[hd + i]);
       }
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-      const float rn = 1.0f / sqrtf(ss + unit_eps);
-      for (int i = lane; i < DP; i += kWave) {
-        float rv = 0.f, kv = 0.f, wv = 0.f, av = 0.f;
-        if (i < d) {
-          rv = lds<T>(sr + r0 + hd + i);
-          kv = lds<T>(sr + k0 + hd + i);
-          wv = expf(-decay_scale *
-                    sigmoid_a(lds<T>(wl + row * (int64_t)(H * d) + hd + i) +
-                              w0[hd + i]));
-          av = sigmoid_a(lds<T>(sr + a0 + hd + i) + ab[hd + i]);
-        }
-        const float uv = kv * rn;
-        sR[tt * DP + i] = rv;
-        sK[tt * DP + i] = kv;
-        sW[tt * DP + i] = wv;
-        sU[tt * DP + i] = uv;
-        sAU[tt * DP + i] = av * uv;
-      }
+      const int at = tt * DP + padded<R>(i);
+      sR[at] = rv;
+      sK[at] = kv;
+      sW[at] = wv;
+      sAK[at] = av * kv;
     }
     for (int idx = threadIdx.x; idx < tc * JB; idx += blockDim.x) {
       const int tt = idx / JB, c = idx % JB;
@@ -320,28 +428,41 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
                     : 0.f;
     }
     __syncthreads();
-    for (int tt = 0; tt < tc; ++tt) {
-      const int base = tt * DP + sl * kRows;
-      const float4* up = reinterpret_cast<const float4*>(sU + base);
-      float us = 0.f;                           // (u^T S)_j over my rows
+    // unit key: u = k * rsqrt(sum k^2 + eps); the update needs u u^T only,
+    // so one scalar 1 / (sum k^2 + eps) per token is enough
+    for (int tt = wid; tt < tc; tt += nw) {
+      float ss = 0.f;
+      for (int i = lane; i < d; i += kWave) {
+        const float kv = sK[tt * DP + padded<R>(i)];
+        ss += kv * kv;
+      }
 #pragma unroll
-      for (int r4 = 0; r4 < kRows / 4; ++r4) {
-        const float4 uv = up[r4];
-        us = fmaf(uv.x, S[4 * r4 + 0], us);
-        us = fmaf(uv.y, S[4 * r4 + 1], us);
-        us = fmaf(uv.z, S[4 * r4 + 2], us);
-        us = fmaf(uv.w, S[4 * r4 + 3], us);
+      for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      if (lane == 0) sRn[tt] = 1.0f / (ss + unit_eps);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < tc; ++tt) {
+      const int base = tt * DP + sl * (R + 4);
+      const float4* kp = reinterpret_cast<const float4*>(sK + base);
+      float ks = 0.f;                           // (k^T S)_j over my rows
+#pragma unroll
+      for (int r4 = 0; r4 < R / 4; ++r4) {
+        const float4 kv = kp[r4];
+        ks = fmaf(kv.x, S[4 * r4 + 0], ks);
+        ks = fmaf(kv.y, S[4 * r4 + 1], ks);
+        ks = fmaf(kv.z, S[4 * r4 + 2], ks);
+        ks = fmaf(kv.w, S[4 * r4 + 3], ks);
       }
       for (int off = NS >> 1; off > 0; off >>= 1)
-        us += __shfl_xor(us, off, 64);
+        ks += __shfl_xor(ks, off, 64);
+      const float us = ks * sRn[tt];            // (a u)(u^T S) = a k * us
       const float vj = sV[tt * JB + jl];
       const float4* wp = reinterpret_cast<const float4*>(sW + base);
-      const float4* ap = reinterpret_cast<const float4*>(sAU + base);
-      const float4* kp = reinterpret_cast<const float4*>(sK + base);
+      const float4* ap = reinterpret_cast<const float4*>(sAK + base);
       const float4* rp = reinterpret_cast<const float4*>(sR + base);
       float acc = 0.f;
 #pragma unroll
-      for (int r4 = 0; r4 < kRows / 4; ++r4) {
+      for (int r4 = 0; r4 < R / 4; ++r4) {
         const float4 wv = wp[r4], av = ap[r4], kv = kp[r4], rv = rp[r4];
         S[4 * r4 + 0] = fmaf(wv.x, S[4 * r4 + 0], fmaf(kv.x, vj, -av.x * us));
         S[4 * r4 + 1] = fmaf(wv.y, S[4 * r4 + 1], fmaf(kv.y, vj, -av.y * us));
@@ -360,8 +481,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   }
   if (col_ok) {
 #pragma unroll
-    for (int r = 0; r < kRows; ++r) {
-      const int row = sl * kRows + r;
+    for (int r = 0; r < R; ++r) {
+      const int row = sl * R + r;
       if (row < d) sp[(int64_t)row * d + j] = S[r];
     }
   }
@@ -388,14 +509,25 @@ Geo make_geo(const torch::Tensor& pos, const c10::optional<torch::Tensor>& lens,
   return g;
 }
 
-// columns x slices of a scan block: slices = 32-row groups (power of two so
-// the lane shuffles pair them up), columns fill the block up to 256 threads
-void scan_shape(int rows, int cols, int& NS, int& JB) {
-  NS = 1;
-  while (NS * kRows < rows) NS *= 2;
-  JB = 1;
-  while (JB < cols && JB * 2 * NS <= 256) JB *= 2;
-  while (JB * NS < kWave) JB *= 2;   // whole waves (spare columns sit idle)
+// Shape of a scan block: R state rows per thread, NS = slices per column (a
+// power of two so lane shuffles pair them up), JB columns so that the block
+// has at most 256 threads and at least one whole wave (spare columns idle).
+// R shrinks from 32 while the launch would leave most SIMDs with one wave.
+void scan_shape(int rows, int cols, int64_t heads_x_batch, int min_r, int& R,
+                int& NS, int& JB) {
+  R = 32;
+  while (R > 8 && R / 2 >= rows) R /= 2;      // no more rows than the state has
+  min_r = min_r < R ? min_r : R;
+  for (;; R /= 2) {
+    NS = 1;
+    while (NS * R < rows) NS *= 2;
+    JB = 1;
+    while (JB < cols && JB * 2 * NS <= 256) JB *= 2;
+    while (JB * NS < kWave) JB *= 2;
+    const int64_t waves =
+        heads_x_batch * ((cols + JB - 1) / JB) * (JB * NS / kWave);
+    if (R <= min_r || waves >= 4096) break;
+  }
 }
 
 }  // namespace
@@ -462,23 +594,37 @@ void causal_conv_silu(torch::Tensor x, int64_t col0, torch::Tensor w,
   if (M == 0) return;
   const Geo g = make_geo(pos, lens, slots, B, T, state.size(0));
   auto st = current_stream();
-  const dim3 grid((unsigned)((C + 255) / 256), (unsigned)M);
+  const bool v4 = C % 4 == 0 && col0 % 4 == 0 && x.size(1) % 4 == 0;
+  const int cpt = v4 ? 4 : 1;                 // channels per thread
+  const dim3 grid((unsigned)((C + 256 * cpt - 1) / (256 * cpt)), (unsigned)M);
   const dim3 sgrid((unsigned)((C + 255) / 256), (unsigned)B);
-#define CV(TT)                                                              \
+  const int ntile = (int)((T + kConvTile - 1) / kConvTile);
+  const dim3 tgrid(grid.x, (unsigned)(B * ntile));
+#define CVT(TT, WW, TP)                                                     \
+  hipLaunchKernelGGL((conv_silu_tile_kernel<TT, WW, TP>), tgrid, dim3(256), \
+                     0, st, (const TT*)x.data_ptr(), x.size(1), (int)col0,  \
+                     w.data_ptr<float>(), bias.data_ptr<float>(),           \
+                     (const TT*)state.data_ptr(), y.data_ptr<float>(), g, C)
+#define CV(TT, WW)                                                          \
   do {                                                                      \
-    hipLaunchKernelGGL((conv_silu_kernel<TT>), grid, dim3(256), 0, st,      \
-                       (const TT*)x.data_ptr(), x.size(1), (int)col0,       \
-                       w.data_ptr<float>(), bias.data_ptr<float>(),         \
-                       (const TT*)state.data_ptr(), y.data_ptr<float>(), g, \
-                       C, taps);                                            \
+    if (taps == 4) CVT(TT, WW, 4);                                          \
+    else if (taps == 3) CVT(TT, WW, 3);                                     \
+    else if (taps == 2) CVT(TT, WW, 2);                                     \
+    else                                                                    \
+      hipLaunchKernelGGL((conv_silu_kernel<TT, WW>), grid, dim3(256), 0,    \
+                         st, (const TT*)x.data_ptr(), x.size(1), (int)col0, \
+                         w.data_ptr<float>(), bias.data_ptr<float>(),       \
+                         (const TT*)state.data_ptr(), y.data_ptr<float>(),  \
+                         g, C, taps);                                       \
     if (taps > 1)                                                           \
       hipLaunchKernelGGL((conv_state_kernel<TT>), sgrid, dim3(256), 0, st,  \
                          (const TT*)x.data_ptr(), x.size(1), (int)col0,     \
                          (TT*)state.data_ptr(), g, C, taps);                \
   } while (0)
-  if (is_bf16(x)) CV(short);
-  else if (is_f32(x)) CV(float);
+  if (is_bf16(x)) { if (v4) CV(short, 4); else CV(short, 1); }
+  else if (is_f32(x)) { if (v4) CV(float, 4); else CV(float, 1); }
   else DNET_CHECK(false, "causal_conv_silu: dtype");
+#undef CVT
 #undef CV
 }
 
@@ -509,25 +655,34 @@ void ssd_scan(torch::Tensor xbc, torch::Tensor dt_src, int64_t dt_col0,
                  y.size(1) == inner, "y fp32 [B*T, heads*P]");
   if (M == 0) return;
   const Geo g = make_geo(pos, lens, slots, B, T, state.size(0));
-  int NS, JB;
-  scan_shape((int)N, (int)P, NS, JB);
-  const int NP = NS * kRows;
-  int TC = 16;
+  int R, NS, JB;
+  // 32 rows per thread: narrower slices multiply the per-token LDS reads of
+  // B and C, which the columns of a wave share (measured slower)
+  scan_shape((int)N, (int)P, heads * B, 32, R, NS, JB);
+  const int NP = NS * (R + 4);
+  int TC = 32;
   while (TC > 1 && (size_t)TC * (2 * NP + JB + 2) * 4 > 48 * 1024) TC /= 2;
   const size_t lds_bytes = (size_t)TC * (2 * NP + JB + 2) * sizeof(float);
   const dim3 grid((unsigned)(heads * ((P + JB - 1) / JB)), (unsigned)B);
   auto st = current_stream();
-#define SS(TD)                                                               \
-  hipLaunchKernelGGL((ssd_scan_kernel<TD>), grid, dim3(JB * NS), lds_bytes,  \
-                     st, xbc.data_ptr<float>(),                              \
+#define SS(TD, RR)                                                           \
+  hipLaunchKernelGGL((ssd_scan_kernel<TD, RR>), grid, dim3(JB * NS),         \
+                     lds_bytes, st, xbc.data_ptr<float>(),                   \
                      (const TD*)dt_src.data_ptr(), dt_src.size(1),           \
                      (int)dt_col0, dt_bias.data_ptr<float>(),                \
                      a_log.data_ptr<float>(), dskip.data_ptr<float>(),       \
                      state.data_ptr<float>(), y.data_ptr<float>(), g,        \
                      (int)heads, (int)P, (int)N, (int)G, JB, NS, TC)
-  if (is_bf16(dt_src)) SS(short);
-  else if (is_f32(dt_src)) SS(float);
+#define SS_R(TD)                          \
+  do {                                    \
+    if (R == 32) SS(TD, 32);              \
+    else if (R == 16) SS(TD, 16);         \
+    else SS(TD, 8);                       \
+  } while (0)
+  if (is_bf16(dt_src)) SS_R(short);
+  else if (is_f32(dt_src)) SS_R(float);
   else DNET_CHECK(false, "ssd_scan: dt dtype");
+#undef SS_R
 #undef SS
 }
 
@@ -558,25 +713,32 @@ void delta_scan(torch::Tensor src, int64_t r0, int64_t k0, int64_t v0,
                  o.size(1) == n, "o fp32 [B*T, H*d]");
   if (M == 0) return;
   const Geo g = make_geo(pos, lens, slots, B, T, state.size(0));
-  int NS, JB;
-  scan_shape((int)d, (int)d, NS, JB);
-  const int DP = NS * kRows;
-  int TC = 16;
-  while (TC > 1 && (size_t)TC * (5 * DP + JB) * 4 > 48 * 1024) TC /= 2;
-  const size_t lds_bytes = (size_t)TC * (5 * DP + JB) * sizeof(float);
+  int R, NS, JB;
+  scan_shape((int)d, (int)d, H * B, 8, R, NS, JB);
+  const int DP = NS * (R + 4);
+  int TC = 32;
+  while (TC > 1 && (size_t)TC * (4 * DP + JB + 1) * 4 > 48 * 1024) TC /= 2;
+  const size_t lds_bytes = (size_t)TC * (4 * DP + JB + 1) * sizeof(float);
   const dim3 grid((unsigned)(H * ((d + JB - 1) / JB)), (unsigned)B);
   auto st = current_stream();
-#define DS(TT)                                                               \
-  hipLaunchKernelGGL((delta_scan_kernel<TT>), grid, dim3(JB * NS),           \
+#define DS(TT, RR)                                                           \
+  hipLaunchKernelGGL((delta_scan_kernel<TT, RR>), grid, dim3(JB * NS),       \
                      lds_bytes, st, (const TT*)src.data_ptr(), src.size(1),  \
                      (int)r0, (int)k0, (int)v0, (int)a0,                     \
                      (const TT*)wl.data_ptr(), w0.data_ptr<float>(),         \
                      ab.data_ptr<float>(), state.data_ptr<float>(),          \
                      o.data_ptr<float>(), g, (int)H, (int)d, JB, NS, TC,     \
                      (float)decay_scale, (float)unit_eps)
-  if (is_bf16(src)) DS(short);
-  else if (is_f32(src)) DS(float);
+#define DS_R(TT)                          \
+  do {                                    \
+    if (R == 32) DS(TT, 32);              \
+    else if (R == 16) DS(TT, 16);         \
+    else DS(TT, 8);                       \
+  } while (0)
+  if (is_bf16(src)) DS_R(short);
+  else if (is_f32(src)) DS_R(float);
   else DNET_CHECK(false, "delta_scan: dtype");
+#undef DS_R
 #undef DS
 }
 
