@@ -151,6 +151,30 @@ __global__ __launch_bounds__(256) void xielu_kernel(
   }
 }
 
+// a channel pair (2i, 2i+1) as one 4 B (bf16) or 8 B (fp32) access
+template <typename T>
+__device__ __forceinline__ void ld_pair(const T* p, float& a, float& b);
+template <> __device__ __forceinline__ void ld_pair<float>(const float* p, float& a, float& b) {
+  const float2 t = *reinterpret_cast<const float2*>(p);
+  a = t.x; b = t.y;
+}
+template <> __device__ __forceinline__ void ld_pair<short>(const short* p, float& a, float& b) {
+  const unsigned t = *reinterpret_cast<const unsigned*>(p);
+  union { unsigned u; float f; } lo, hi;
+  lo.u = t << 16;
+  hi.u = t & 0xffff0000u;
+  a = lo.f; b = hi.f;
+}
+template <typename T>
+__device__ __forceinline__ void st_pair(T* p, float a, float b);
+template <> __device__ __forceinline__ void st_pair<float>(float* p, float a, float b) {
+  *reinterpret_cast<float2*>(p) = make_float2(a, b);
+}
+template <> __device__ __forceinline__ void st_pair<short>(short* p, float a, float b) {
+  *reinterpret_cast<unsigned*>(p) =
+      (unsigned)(unsigned short)f2bits(a) | ((unsigned)(unsigned short)f2bits(b) << 16);
+}
+
 constexpr int kMaxRot = 128;   // rotated pairs per head (head size <= 256)
 
 // qkv row layout: [q: nq*d | k: nkv*d | v: nkv*dv]. Token (b,t) = row b*T+t
@@ -165,7 +189,7 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
     const float eps, const int nq, const int nkv, const int d, const int dv,
     const int Tn, const int Bc, const int Hkv, const int Smax,
     const bool per_head, const float* __restrict__ rot_freq,
-    const int nrot) {
+    const int nrot, const bool pairs) {
   __shared__ float red[8];
   const int64_t row = blockIdx.x;
   const int b = (int)(row / Tn);
@@ -234,8 +258,13 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
 #pragma unroll
         for (int qd = 0; qd < 2; ++qd) {
           const int e0 = 2 * (lane + kWave * qd);
-          v0[qd] = e0 < d ? ldf<T>(hs + e0) : 0.f;
-          v1[qd] = e0 + 1 < d ? ldf<T>(hs + e0 + 1) : 0.f;
+          v0[qd] = v1[qd] = 0.f;
+          if (pairs) {                // d even, rows pair-aligned (uniform)
+            if (e0 < d) ld_pair<T>(hs + e0, v0[qd], v1[qd]);
+          } else {
+            if (e0 < d) v0[qd] = ldf<T>(hs + e0);
+            if (e0 + 1 < d) v1[qd] = ldf<T>(hs + e0 + 1);
+          }
           ss += v0[qd] * v0[qd] + v1[qd] * v1[qd];
         }
 #pragma unroll
@@ -255,8 +284,12 @@ __global__ __launch_bounds__(256) void qknorm_append_kernel(
             a1 = a1 * cs + a0 * sn;
             a0 = u0;
           }
-          stf<T>(dst + e0, a0);
-          if (e1 < d) stf<T>(dst + e1, a1);
+          if (pairs) {
+            st_pair<T>(dst + e0, a0, a1);
+          } else {
+            stf<T>(dst + e0, a0);
+            if (e1 < d) stf<T>(dst + e1, a1);
+          }
         }
         continue;
       }
@@ -413,6 +446,53 @@ __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(
     v = v * r * wr[e];
     if (!gate_first) v *= gv;
     stf<TO>(orow + e, v);
+  }
+}
+
+// Wide groups (>= 1024 channels): one workgroup per (row, group), 4-wide
+// accesses when the group size and the gate's stride and offset allow.
+template <typename TG, typename TO, int W>
+__global__ __launch_bounds__(256) void gated_group_rmsnorm_wide_kernel(
+    const float* __restrict__ y, const TG* __restrict__ gate_src,
+    const int64_t gld, const int gcol0, const float* __restrict__ w,
+    TO* __restrict__ out, const int N, const int groups, const float eps,
+    const bool gate_silu, const bool gate_first) {
+  __shared__ float red[8];
+  const int64_t row = blockIdx.y;
+  const int grp = blockIdx.x;
+  const int gs = N / groups;
+  const float* yr = y + row * N + (int64_t)grp * gs;
+  const TG* gr = gate_src + row * gld + gcol0 + (int64_t)grp * gs;
+  float ss = 0.f;
+  for (int e = threadIdx.x * W; e < gs; e += blockDim.x * W) {
+    vecf<W> v = ldw<W, float>(yr + e);
+    if (gate_first) {
+      const vecf<W> g = ldw<W, TG>(gr + e);
+#pragma unroll
+      for (int j = 0; j < W; ++j)
+        v.v[j] *= gate_silu ? g.v[j] * sigmoid_f(g.v[j]) : sigmoid_f(g.v[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < W; ++j) ss += v.v[j] * v.v[j];
+  }
+  ss = block_reduce_sum(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)gs + eps);
+  TO* orow = out + row * N + (int64_t)grp * gs;
+  const float* wr = w + (int64_t)grp * gs;
+  for (int e = threadIdx.x * W; e < gs; e += blockDim.x * W) {
+    vecf<W> v = ldw<W, float>(yr + e);
+    const vecf<W> g = ldw<W, TG>(gr + e), wv = ldw<W, float>(wr + e);
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+      const float gv =
+          gate_silu ? g.v[j] * sigmoid_f(g.v[j]) : sigmoid_f(g.v[j]);
+      float t = v.v[j];
+      if (gate_first) t *= gv;
+      t = t * r * wv.v[j];
+      if (!gate_first) t *= gv;
+      v.v[j] = t;
+    }
+    stw<W, TO>(orow + e, v);
   }
 }
 
@@ -626,8 +706,11 @@ void qknorm_append(torch::Tensor qkv, torch::Tensor qw, torch::Tensor kw,
                      (int)nq, (int)nkv, (int)d, (int)dv, (int)T, Bc, Hkv,     \
                      Smax,                                                   \
                      per_head, nrot ? rot_freq->data_ptr<float>() : nullptr, \
-                     nrot)
+                     nrot, pairs)
   const bool v4 = d % 4 == 0 && dv % 4 == 0;
+  // per-head path: channel pairs as single accesses when every head starts
+  // on a pair boundary in the projection row, in q and in the cache
+  const bool pairs = d % 2 == 0 && qkv.size(1) % 2 == 0;
   if (is_bf16(qkv)) { if (v4) QA(short, 4); else QA(short, 1); }
   else if (is_f32(qkv)) { if (v4) QA(float, 4); else QA(float, 1); }
   else DNET_CHECK(false, "qknorm_append: dtype");
@@ -702,19 +785,34 @@ void gated_group_rmsnorm(torch::Tensor y, torch::Tensor gate_src,
              "out [M, N]");
   if (M == 0) return;
   auto st = current_stream();
-  const dim3 grid((unsigned)((groups + 3) / 4), (unsigned)M);
+  const int gs = N / (int)groups;
+  const bool wide = gs >= 1024;
+  const bool v4 = gs % 4 == 0 && gate_src.size(1) % 4 == 0 && gate_col0 % 4 == 0;
+  const dim3 grid(wide ? (unsigned)groups : (unsigned)((groups + 3) / 4),
+                  (unsigned)M);
+#define GG_ARGS(TG, TO)                                                      \
+  grid, dim3(256), 0, st, y.data_ptr<float>(),                               \
+      (const TG*)gate_src.data_ptr(), gate_src.size(1), (int)gate_col0,      \
+      w.data_ptr<float>(), (TO*)out.data_ptr(), N, (int)groups, (float)eps,  \
+      gate_silu, gate_first
 #define GG(TG, TO)                                                           \
-  hipLaunchKernelGGL((gated_group_rmsnorm_kernel<TG, TO>), grid, dim3(256),  \
-                     0, st, y.data_ptr<float>(),                             \
-                     (const TG*)gate_src.data_ptr(), gate_src.size(1),       \
-                     (int)gate_col0, w.data_ptr<float>(),                    \
-                     (TO*)out.data_ptr(), N, (int)groups, (float)eps,        \
-                     gate_silu, gate_first)
+  do {                                                                       \
+    if (wide && v4)                                                          \
+      hipLaunchKernelGGL((gated_group_rmsnorm_wide_kernel<TG, TO, 4>),       \
+                         GG_ARGS(TG, TO));                                   \
+    else if (wide)                                                           \
+      hipLaunchKernelGGL((gated_group_rmsnorm_wide_kernel<TG, TO, 1>),       \
+                         GG_ARGS(TG, TO));                                   \
+    else                                                                     \
+      hipLaunchKernelGGL((gated_group_rmsnorm_kernel<TG, TO>),               \
+                         GG_ARGS(TG, TO));                                   \
+  } while (0)
   if (is_bf16(gate_src) && is_bf16(out)) GG(short, short);
   else if (is_f32(gate_src) && is_f32(out)) GG(float, float);
   else if (is_bf16(gate_src) && is_f32(out)) GG(short, float);
   else if (is_f32(gate_src) && is_bf16(out)) GG(float, short);
   else DNET_CHECK(false, "gated_group_rmsnorm: dtypes");
+#undef GG_ARGS
 #undef GG
 }
 

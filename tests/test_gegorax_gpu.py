@@ -174,7 +174,9 @@ def test_delta_scan(dt, H, d):
 @pytest.mark.parametrize("silu,first,groups,N", [(True, True, 2, 128),
                                                  (False, False, 3, 60),
                                                  (True, False, 1, 200),
-                                                 (False, True, 8, 64)])
+                                                 (False, True, 8, 64),
+                                                 (True, True, 1, 2048),
+                                                 (False, False, 2, 2050)])
 def test_gated_group_rmsnorm(dt, silu, first, groups, N):
     torch.manual_seed(N)
     M = 9
