@@ -566,6 +566,45 @@ def test_other_sizes(device, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mid_size_long_prompt(dtype, device="cuda:0"):
+    """(GPU only: the reference ops walk the recurrences token by token in
+    Python.) Head sizes of 48 to 128, state sizes of 16 to 128, several pooled
+    chunks and windows that pass over prompt and decoded tokens: two unequal
+    prompts in position chunks, then decoding together and alone."""
+    layers = [
+        (delta(3, 96), dense(300)),
+        (par(heads=8, kv=4, dim=64, vdim=32, size=100, pool=5, rot=32,
+             base=1e4, sh=6, svd=48, state=64, groups=3, ng=3, conv=3),
+         moe(experts=10, top=3, ff=72, limit=1.1, shared=40, slimit=0.9)),
+        (par(heads=6, kv=1, dim=80, vdim=112, size=37, pool=8, rot=80,
+             base=3e3, sh=4, svd=64, state=128, groups=2, ng=1, conv=4),
+         dense(520)),
+        (delta(5, 48), moe(experts=6, top=2, ff=64, limit=2.0, shared=0)),
+        (par(heads=4, kv=2, dim=128, vdim=128, size=64, pool=16, rot=64,
+             base=2e4, sh=8, svd=32, state=16, groups=4, ng=2, conv=2), None),
+    ]
+    cfg = make_cfg(layers, width=256, vocab=300, eps=1e-6, side=20)
+    sd = make_weights(cfg, 77, rank=12, dtype=dtype)
+    a, b = tokens(230, 300, 1), tokens(100, 300, 2)
+    wa, wb = oracle(a, cfg, sd), oracle(b, cfg, sd)
+    ex = executor(cfg, sd, device, dtype, slots=4, smax=320)
+    na, nb = 215, 90
+    got = ex.prefill_slots([3, 1], [a[:na], b[:nb]],
+                           want=[list(range(0, na, 7)), list(range(0, nb, 5))],
+                           chunk=96)
+    close(got[0], wa[0:na:7], dtype)
+    close(got[1], wb[0:nb:5], dtype)
+    for i in range(10):
+        lg = decode_steps(ex, {3: a[na + i], 1: b[nb + i]})
+        close(lg[3:4], wa[na + i].view(1, -1), dtype)
+        close(lg[1:2], wb[nb + i].view(1, -1), dtype)
+    for i in range(10, 15):                 # the shorter request has ended
+        lg = decode_steps(ex, {3: a[na + i]})
+        close(lg[3:4], wa[na + i].view(1, -1), dtype)
+
+
+@pytest.mark.gpu
 def test_decode_graph_replays_match_eager():
     """Captured decode steps, replayed with eager prefills and host syncs in
     between, equal the eager steps every time (warm-up runs of the capture
