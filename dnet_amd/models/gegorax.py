@@ -66,7 +66,9 @@ class GegoraxRingModel(RingModel):
     act_dtype = torch.float32          # residual stream / ring hops
     ragged_prefill = True
     supports_float32 = True
-    needs_tokens = True                # layers read the token ids again
+    # layers read the token ids again: the executor calls set_tokens on
+    # every pipeline stage
+    needs_tokens = True
     stateful = True                    # idle decode rows must not step
     DENSE_MOE_MAX_T = 64
 

@@ -123,12 +123,12 @@ class RingExecutor:
                              self.is_last, smax=smax, tp_rank=self.tp_rank,
                              tp_size=tp, tp_group=stage_group)
         self.model.kv_bits = kv_bits
-        if getattr(self.model, "needs_tokens", False) and self.stages > 1:
-            # the ring hops carry the residual only; layers that read the
-            # token ids again need them on every stage
-            raise NotImplementedError(
-                f"{cfg.model_type}: pipeline stages are not implemented "
-                "(every layer reads the token ids)")
+        # families whose layers read the token ids again: the ring hops
+        # carry the residual only, so every stage is handed the ids of the
+        # rows it runs (prompts are given to every rank; step tokens reach
+        # every rank through the token broadcast)
+        self._needs_tokens = bool(getattr(self.model, "needs_tokens", False))
+        self._tok_all = self._needs_tokens and self.stages > 1
         if init_weights:
             self.model.init_random(seed)
         self.weight_cache = None
@@ -228,6 +228,8 @@ class RingExecutor:
     def _decode_body(self, mb: int, r: int = 0):
         if self.is_first and r == 0:
             self.hbuf[mb].copy_(self.model.embed_tokens(self.tokbuf[mb]))
+        elif self._needs_tokens:
+            self.model.set_tokens(self.tokbuf[mb])
         if self.windows[r]:
             self.model.decode_window(self.hbuf[mb], self.windows[r],
                                      self.kvs[mb])
@@ -314,7 +316,9 @@ class RingExecutor:
 
         ``chunk`` > 0 prefills in position chunks of that size (row-wise
         identical math — same tokens — while bounding the activation
-        buffer to [B, chunk, H] for long prompts)."""
+        buffer to [B, chunk, H] for long prompts). Families whose layers
+        read the token ids (``needs_tokens``) take the real tokens on
+        every rank."""
         M, B, T = tokens.shape
         assert M == self.mb_count and B == self.mb_size
         H = self.cfg.hidden_size
@@ -336,6 +340,9 @@ class RingExecutor:
                                             dtype=self.model.act_dtype,
                                             device=self.device)
                         self.ring.recv(h)
+                        if self._needs_tokens:
+                            self.model.set_tokens(
+                                tokens[mb, :, p0:p1].to(self.device))
                     if self.windows[r]:
                         self.model.prefill_window(h, self.windows[r],
                                                   self.kvs[mb], p0)
@@ -357,6 +364,12 @@ class RingExecutor:
                     # (single-stage TP: is_first too, so no self-send)
         for r in tok_reqs:
             r.wait()
+        if self._tok_all:
+            # every stage needs the step tokens: hand the first ones round
+            for mb in range(M):
+                dist.broadcast(first_tokens[mb],
+                               src=(self.stages - 1) * self.tp)
+                self.tokbuf[mb].copy_(first_tokens[mb])
         if self.is_first:
             for mb in range(M):
                 self.tokbuf[mb].copy_(first_tokens[mb])
@@ -368,6 +381,11 @@ class RingExecutor:
 
         Returns generated tokens [mb_count, mb_size, n] on rank 0, else None.
         rank 0's tokbuf must hold the current token (set by prefill)."""
+        if self._tok_all:
+            # this schedule returns sampled tokens to the first stage only
+            raise NotImplementedError(
+                "decode_rounds: families that read the token ids on every "
+                "stage decode through decode_stream / the slot steps")
         M = self.mb_count
         out = (torch.zeros(M, self.mb_size, n, dtype=torch.int64,
                            device=self.device) if (collect and self.is_first)
@@ -478,8 +496,10 @@ class RingExecutor:
         whose logits are returned (default: its last). ``start[i]``: tokens
         slot i already holds (default 0: a fresh request); the prompt then
         continues from there. Position-chunked by ``chunk`` to bound
-        activations. Returns a list of logits
-        [len(want[i]), V] on the LAST stage, else None."""
+        activations. Families whose layers read the token ids take the
+        real prompts on every rank (the serving runtime broadcasts them).
+        Returns a list of logits [len(want[i]), V] on the LAST stage, else
+        None."""
         n = len(slots)
         lens = [int(p.shape[-1]) for p in prompts]
         if want is None:
@@ -524,6 +544,9 @@ class RingExecutor:
                                             dtype=self.model.act_dtype,
                                             device=self.device)
                         self.ring.recv(h)
+                        if self._needs_tokens:
+                            self.model.set_tokens(
+                                tok[:, p0:p1].to(self.device))
                     if self.windows[r]:
                         if self.model.ragged_prefill:
                             self.model.prefill_window(

@@ -762,14 +762,66 @@ def test_trace_replay_cli(tmp_path, dtype="float32"):
     close(rd(6), torch.stack([w["c"][11], w["d"][5]]), dtype)
 
 
-def test_pipeline_stages_are_refused():
-    """Every layer reads the token ids; the ring hops carry the residual
-    only, so a second stage is refused at construction."""
+# ---------- pipeline stages (gloo, two processes) ----------
+
+def _ring_tokens():
+    g = torch.Generator().manual_seed(21)
+    return torch.randint(0, 83, (1, 2, 13), generator=g)
+
+
+def _ring_run(rank, world):
     mc = ModelConfig.from_hf(make_cfg(BASE))
-    from dnet_amd.parallel.ring import RingPlan
-    with pytest.raises(NotImplementedError):
-        RingExecutor(mc, 0, 2, "cpu", plan=RingPlan.contiguous(4, 2),
-                     init_weights=False, use_graphs=False)
+    mc.compute_dtype = "float32"
+    ex = RingExecutor(mc, rank, world, "cpu", mb_count=1, mb_size=2, smax=64,
+                      seed=7, use_graphs=False)
+    first = ex.prefill(_ring_tokens(), chunk=5)
+    steps = []
+    ex.decode_stream(6, on_token=lambda s, t, last: steps.append(t.clone()))
+    if world > 1:
+        with pytest.raises(NotImplementedError):
+            ex.decode_rounds(1)
+    if rank:
+        return None
+    return torch.cat([first.view(2, 1)] + [t.view(2, 1) for t in steps], -1)
+
+
+def _ring_rank_main(rank, world, port, q):
+    import os
+    os.environ.update(RANK=str(rank), WORLD_SIZE=str(world),
+                      MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port),
+                      LOCAL_RANK=str(rank))
+    import torch.distributed as dist
+    dist.init_process_group("gloo", rank=rank, world_size=world)
+    out = _ring_run(rank, world)
+    if rank == 0:
+        q.put(out)
+    dist.destroy_process_group()
+
+
+@pytest.mark.timeout(360)
+def test_two_stage_ring_matches_single():
+    """Layers split over two pipeline stages: the fp32 residual rides the
+    ring hops, every stage is handed the token ids its layers read again
+    (prompt on every rank, step tokens through the broadcast), and the
+    generated tokens equal the single-stage run."""
+    import multiprocessing as mp
+    import socket
+    single = _ring_run(0, 1)
+    s = socket.socket()
+    s.bind(("127.0.0.1", 0))
+    port = s.getsockname()[1]
+    s.close()
+    ctx = mp.get_context("spawn")
+    q = ctx.Queue()
+    procs = [ctx.Process(target=_ring_rank_main, args=(r, 2, port, q))
+             for r in range(2)]
+    for p in procs:
+        p.start()
+    out = q.get(timeout=200)
+    for p in procs:
+        p.join(timeout=60)
+        assert p.exitcode == 0
+    assert single.shape == (2, 6) and torch.equal(out, single)
 
 
 def test_synthetic_preset_runs():
