@@ -509,3 +509,17 @@ class GegoraxRingModel(RingModel):
         y = ops.rmsnorm_rows(h, self.final_norm, self.cfg.rms_eps,
                              self.wdtype)
         return self.lm_head(y)
+
+    def weight_bytes(self) -> int:
+        """Bytes of every tensor and linear the resident layers hold (the
+        layer kinds carry different sets of them)."""
+        def size(v) -> int:
+            if isinstance(v, Linear):
+                return v.nbytes()
+            if torch.is_tensor(v):
+                return v.numel() * v.element_size()
+            if isinstance(v, (list, tuple)):
+                return sum(size(x) for x in v)
+            return 0
+        return sum(size(v) for lw in self.layers.values()
+                   for k, v in vars(lw).items() if k != "experts_stacked")

@@ -15,7 +15,7 @@ from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Iterator, Optional
 
-# "layers.N." (HF layouts) or "lN." (posudra layout)
+# "layers.N." (HF layouts) or "lN." (posudra / gegorax layout)
 _LAYER_RE = re.compile(r"^(?:model\.)?(?:layers\.|l)(\d+)\.(.+)$")
 _DTYPE_BYTES = {"F64": 8, "F32": 4, "F16": 2, "BF16": 2, "I64": 8, "I32": 4,
                 "I16": 2, "I8": 1, "U8": 1, "BOOL": 1, "F8_E4M3": 1,
