@@ -70,6 +70,7 @@ class GegoraxRingModel(RingModel):
     # every pipeline stage
     needs_tokens = True
     stateful = True                    # idle decode rows must not step
+    supports_offload = False           # layer kinds hold different tensors
     DENSE_MOE_MAX_T = 64
 
     def __init__(self, cfg: ModelConfig, layer_ids: Sequence[int], device,

@@ -63,6 +63,10 @@ def enable_offload(model: RingModel, residency: int,
     layers must share one tensor-shape template (true for uniform stacks —
     deepseek's mixed dense/MoE stack is not offloadable yet)."""
     assert model.layers, "load or init weights first"
+    if not getattr(model, "supports_offload", True):
+        raise NotImplementedError(
+            f"{model.model_type}: windowed weight residency is not "
+            "implemented (its layer kinds hold different tensor sets)")
     group = model.cfg.quant.group if model.cfg.quant else 0
     packed = False
     # group layers by tensor-shape template: the LARGEST uniform group

@@ -824,6 +824,16 @@ def test_two_stage_ring_matches_single():
     assert single.shape == (2, 6) and torch.equal(out, single)
 
 
+def test_weight_streaming_is_refused():
+    """The layer kinds hold different tensor sets, which the windowed weight
+    cache's one-template slots cannot stream: asking for it raises."""
+    from dnet_amd.models import PRESETS
+    mc = ModelConfig.from_hf(dict(PRESETS["gegorax-tiny"]))
+    with pytest.raises(NotImplementedError):
+        RingExecutor(mc, 0, 1, "cpu", mb_size=1, smax=32, residency=2,
+                     use_graphs=False)
+
+
 def test_synthetic_preset_runs():
     """The benchmark preset builds with seeded random weights and generates
     the same tokens whatever the slot a prompt sits in."""
